@@ -100,6 +100,28 @@ def test_c4_q8_gemm_phi2_prefill(device, oracle, phi2_up):
     assert got.shape == (1, 512, 2560) and oracle.max_rel_err(got, want) <= 2e-2
 
 
+def test_c4_f16_weights_phi2_prefill(device, oracle):
+    """The metric's f16 GEMM: [512 x 2560] . [10240 x 2560]^T + b with f16 weights, full size, then the
+    down-projection [512 x 10240] . [2560 x 10240]^T; each output against the oracle's f32 GEMM."""
+    rng = np.random.default_rng(4)
+    w = (rng.standard_normal((10240, 2560)) * 0.02).astype(np.float16)
+    bias = rng.standard_normal(10240).astype(np.float16)
+    x = rng.standard_normal((1, 512, 2560)).astype(np.float16)
+    got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x), Tensor.from_data(bias), False, True, True)
+    want = oracle.matmul_ref(w, oracle.F16, w.shape, x, oracle.F16, x.shape, bias, False, True, True)
+    assert got.shape == (1, 512, 10240) and oracle.max_rel_err(got, want) <= 2e-2
+    # the same product spelled from the activation side: x.matmul(W, false, true) + no bias
+    got = gpu_matmul(device, Tensor.from_data(x), Tensor.from_data(w), None, False, True, False)
+    want = oracle.matmul_ref(x, oracle.F16, x.shape, w, oracle.F16, w.shape, None, False, True, False)
+    assert got.shape == (1, 512, 10240) and oracle.max_rel_err(got, want) <= 2e-2
+    wd = (rng.standard_normal((2560, 10240)) * 0.02).astype(np.float16)
+    bd = rng.standard_normal(2560).astype(np.float16)
+    h = rng.standard_normal((1, 512, 10240)).astype(np.float16)
+    got = gpu_matmul(device, Tensor.from_data(wd), Tensor.from_data(h), Tensor.from_data(bd), False, True, True)
+    want = oracle.matmul_ref(wd, oracle.F16, wd.shape, h, oracle.F16, h.shape, bd, False, True, True)
+    assert got.shape == (1, 512, 2560) and oracle.max_rel_err(got, want) <= 2e-2
+
+
 @pytest.mark.parametrize("M", [1, 16, 256])
 def test_c5_q4k_phi3(device, oracle, M):
     rng = np.random.default_rng(5)

@@ -81,6 +81,14 @@ def test_dequantize_q4k_bit_exact(device, oracle):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_dequantize_q4k_known_answer_block(device, q4k_kat):
+    """The hand-typed super-block and its hand-worked values (tests/conftest.py): no packer, no oracle."""
+    blk, want, _ = q4k_kat
+    blocks = np.tile(blk, 3)
+    got = dequantize(Tensor.from_quantized(blocks, DType.Q4_K, (3, 256), device)).to_ndarray()
+    assert np.array_equal(got.view(np.uint32), np.tile(want, (3, 1)).view(np.uint32))
+
+
 @pytest.mark.parametrize("dt", [DType.Q8_0F, DType.Q8_0H])
 def test_transcode_bit_exact(device, oracle, dt):
     f16 = dt == DType.Q8_0H

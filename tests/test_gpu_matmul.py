@@ -629,9 +629,9 @@ def test_q4k_prefill_tiles(device, oracle):
 
 def test_q4k_prefill_one_hot_is_the_dequantized_weight(device, oracle):
     """A one-hot activation row selects one dequantized weight per weight row: the tiled kernel must return
-    d * sc * q - dmin * mn, rounded to f16 once, for every super-block position.  The oracle rounds d * sc and
-    dmin * mn to f32 first (ggml's order) and the kernel rounds d * (sc q) instead, so a value that sits on an f16
-    rounding boundary may land on the neighbouring f16: at most one unit in the last place, and rarely."""
+    d * sc * q - dmin * mn rounded to f32 and then to f16, bit for bit, for every super-block position.
+    d * sc, (d * sc) * q and dmin * mn are exact in f32 (11 + 6 + 4 bits), so the order in which the kernel
+    forms d * (sc * q) cannot matter: only the subtraction rounds, in the oracle and in the kernel alike."""
     rng = np.random.default_rng(1220)
     N, K, M = 150, 1024, 300
     blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
@@ -641,8 +641,33 @@ def test_q4k_prefill_one_hot_is_the_dequantized_weight(device, oracle):
     x[0, np.arange(M), cols] = 1
     got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (N, K)), Tensor.from_data(x), None, False, True, True)
     want = dq[:, cols].T.astype(np.float16)
-    ulps = np.abs(got[0].view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
-    assert ulps.max() <= 1 and np.count_nonzero(ulps) <= got[0].size // 1000, (ulps.max(), np.count_nonzero(ulps))
+    bad = np.argwhere(got[0].view(np.uint16) != want.view(np.uint16))
+    assert bad.size == 0, (len(bad), bad[:8].tolist())
+
+
+@pytest.mark.parametrize("M", [1, 16, 64, 256], ids=["streaming-1", "streaming-16", "tiled-64", "tiled-256"])
+def test_q4k_known_answer_block_through_every_kernel(device, oracle, q4k_kat, M):
+    """The hand-typed known-answer super-block (tests/conftest.py) as a weight: 64 weight rows x 4 super-blocks,
+    every block a copy of it with its f16 d scaled by an exact power of two per (row, block) so that a
+    misplaced block shows.  One-hot activations return single dequantized weights: compared bit for bit
+    with the hand-worked values, not with the oracle."""
+    blk, w, _ = q4k_kat
+    N, NB = 64, 4
+    K = 256 * NB
+    blocks = np.tile(blk, (N, NB, 1))
+    expo = (np.arange(N)[:, None] + 3 * np.arange(NB)[None, :]) % 5          # d, dmin *= 2^-expo
+    for f in (0, 2):                                                          # the two f16 headers: exponent field -= expo
+        h = blocks[:, :, f:f + 2].copy().view(np.uint16)[:, :, 0] - (expo.astype(np.uint16) << 10)
+        blocks[:, :, f:f + 2] = h[:, :, None].view(np.uint8)
+    dense = (w[None, None, :] * (2.0 ** -expo)[:, :, None]).reshape(N, K).astype(np.float32)
+    rng = np.random.default_rng(1230 + M)
+    cols = np.concatenate([np.arange(0, K, 257), rng.integers(0, K, size=M)])[:M]
+    x = np.zeros((1, M, K), dtype=np.float16)
+    x[0, np.arange(M), cols] = 1
+    got = gpu_matmul(device, Tensor.from_quantized(blocks.reshape(-1), DType.Q4_K, (N, K)), Tensor.from_data(x), None,
+                     False, True, True)
+    want = dense[:, cols].T.astype(np.float16)
+    assert np.array_equal(got[0].view(np.uint16), want.view(np.uint16))
 
 
 # ---------------------------------------------------------------------------

@@ -216,6 +216,18 @@ def test_q4k_dequantize_hand_built(oracle):
     assert np.array_equal(got.astype(np.float32), want.astype(np.float32))
 
 
+def test_q4k_known_answer_block(oracle, q4k_kat):
+    """The hand-typed 144 bytes and hand-worked values of tests/conftest.py: independent of _q4k_block above,
+    including the j >= 4 scales and mins whose two high bits live in scales[0..7]."""
+    blk, want, scmn = q4k_kat
+    for j in range(8):
+        assert oracle.q4k_scale_min(j, blk[4:16]) == scmn[j]
+    assert np.array_equal(oracle.q4k_dequantize(blk).view(np.uint32), want.view(np.uint32))
+    # and the packer used by the other tests agrees with the hand-typed bytes
+    nib = np.concatenate([np.array(n + n) for _, _, n in __import__("conftest").Q4K_KAT_SUBBLOCKS])
+    assert np.array_equal(_q4k_block(0.375, 0.625, [s for s, _ in scmn], [m for _, m in scmn], nib), blk)
+
+
 def test_q4k_quantizer_round_trip(oracle):
     rng = np.random.default_rng(7)
     w = (rng.standard_normal(256 * 40) * 0.02).astype(np.float32)
