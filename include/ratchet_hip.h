@@ -328,6 +328,20 @@ RT_API rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, c
                                       const void *bias, void *out, int32_t activation, void *workspace,
                                       uint64_t workspace_bytes, void *stream);
 
+/* rt_matmul_enqueue_ws for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the shares' partial sums go to a static
+ * buffer of RT_STATIC_SCRATCH_BYTES that the library holds on each GPU it runs on, from
+ * rt_ctx_create until the process ends.  Neither this call nor anything it launches allocates or
+ * frees.  Results are those of rt_matmul_enqueue_ws with a workspace of rt_matmul_workspace_bytes,
+ * bit for bit (the same kernels run).  A split that would need more than the buffer holds is
+ * RT_ERR_UNSUPPORTED (on a device of up to 256 compute units none does); a product that is not split
+ * runs as rt_matmul_enqueue_fused and touches no scratch.  All calls on one GPU share the one buffer:
+ * calls that can overlap there (different streams, different contexts or threads) race; order them.
+ * No counterpart in the reference, whose operators never own scratch memory. */
+#define RT_STATIC_SCRATCH_BYTES (20u << 20)
+RT_API rt_status rt_matmul_enqueue_static(rt_ctx *ctx, const rt_matmul_desc *desc, const void *lhs, const void *rhs,
+                                          const void *bias, void *out, int32_t activation, void *stream);
+
 /* Replaces: Unary (ops/unary.rs:71-260) for Gelu and Silu on F32 / F16 tensors; `dst` may be
  * `src` (the reference runs unary operators in place when it can). */
 RT_API rt_status rt_unary_enqueue(rt_ctx *ctx, int32_t activation, int32_t dtype, const void *src, void *dst,

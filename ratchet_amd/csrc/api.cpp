@@ -17,11 +17,22 @@ rt_status gguf_load_tensor(const rt_gguf *g, const void *image, uint64_t size, u
                            void *staging, void *dst, hipStream_t stream, std::string &why, hipError_t &herr);
 }
 
+// Library-owned scratch for rt_matmul_enqueue_static: the f32 partial sums of a product whose K is
+// shared among workgroups.  Every GPU the library runs on holds its own copy of the array at its
+// own address for the life of the process.  A split keeps tiles x shares within the compute-unit
+// count, so on a device of up to 256 compute units no split needs more than 256 tiles of
+// 160 x 128 floats, which is this size.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels are given the address that call returns.
+constexpr uint64_t kStaticScratchBytes = RT_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 struct rt_ctx {
     rt::DeviceInfo dev;
     std::mutex mu;
     std::string last_error;
     int last_hip = 0;
+    void *static_scratch = nullptr;   // device address of `scratch` on this context's GPU
+    hipError_t static_scratch_err = hipSuccess;
 };
 
 namespace {
@@ -157,6 +168,14 @@ rt_status rt_ctx_create(int32_t device_ordinal, rt_ctx **ctx) {
     rt_ctx *c = new rt_ctx();
     c->dev.ordinal = device_ordinal;
     c->dev.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    {
+        // the address of the static scratch array on this GPU (each device has its own copy)
+        DeviceGuard dg(device_ordinal);
+        void *ptr = nullptr;
+        c->static_scratch_err = dg.ok ? hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) : hipErrorInvalidDevice;
+        if (c->static_scratch_err == hipSuccess) c->static_scratch = ptr;
+        else (void)hipGetLastError();
+    }
     *ctx = c;
     return RT_OK;
     RT_GUARD_END(nullptr)
@@ -285,6 +304,24 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
     if (e != hipSuccess) return hip_fail(ctx, "matmul launch", e);
     return RT_OK;
     RT_GUARD_END(ctx)
+}
+
+rt_status rt_matmul_enqueue_static(rt_ctx *ctx, const rt_matmul_desc *desc, const void *lhs, const void *rhs,
+                                   const void *bias, void *out, int32_t activation, void *stream) {
+    if (!ctx || !desc) return RT_ERR_INVALID_ARG;
+    uint64_t need = 0;
+    const rt_status st = rt_matmul_workspace_bytes(ctx, desc, &need);
+    if (st != RT_OK) return st;
+    if (need == 0) // this product is not split: no scratch is touched
+        return rt_matmul_enqueue_ws(ctx, desc, lhs, rhs, bias, out, activation, nullptr, 0, stream);
+    if (need > kStaticScratchBytes)
+        return fail(ctx, RT_ERR_UNSUPPORTED,
+                    "rt_matmul_enqueue_static: the split of this product needs " + std::to_string(need) +
+                        " bytes of scratch, the static buffer holds " + std::to_string(kStaticScratchBytes));
+    if (!ctx->static_scratch)
+        return hip_fail(ctx, "rt_matmul_enqueue_static: hipGetSymbolAddress of the static scratch failed", ctx->static_scratch_err);
+    // every share's sums are written before the second kernel reads them, so nothing needs clearing
+    return rt_matmul_enqueue_ws(ctx, desc, lhs, rhs, bias, out, activation, ctx->static_scratch, kStaticScratchBytes, stream);
 }
 
 rt_status rt_quantize_q8_0(rt_ctx *ctx, const void *src_f32, uint64_t numel, void *dst, void *stream) {
