@@ -81,11 +81,15 @@ class Runner:
             raise RuntimeError(f"rt_matmul_enqueue: {self.ffi.status_string(st)} "
                                f"{self.L.rt_last_error(self.dev.ctx).decode()}")
 
-    def time_steps(self, launch_step, steps, warmup, n_variants):
-        """Times `steps` calls of launch_step(i) after `warmup` untimed ones.  The launches
-        are captured into one HIP graph of whole rotations of the weight copies (20 launches
-        or more) when capture works, so the host's launch rate does not bound a ~4 us kernel; otherwise they
-        are issued one by one.  Returns (ms_per_step, mode)."""
+    REGIONS = 11   # timed regions of `steps` launches each; the median is reported
+
+    def time_steps(self, launch_step, steps, warmup, n_variants, stats=None):
+        """Times `steps` calls of launch_step(i) after `warmup` untimed ones, REGIONS times over, each region
+        between its own pair of HIP events on the launch stream, and returns the median region's
+        (ms_per_step, mode); `stats`, a dict, also receives the fastest and slowest region and the count.
+        The launches are captured into one HIP graph of whole rotations of the weight copies (20 launches
+        or more) when capture works, so the host's launch rate does not bound a ~6 us kernel; a region is
+        steps // 20 replays plus the remaining launches one by one.  Otherwise all are issued one by one."""
         torch = self.torch
         for i in range(warmup):
             launch_step(i % n_variants)
@@ -104,21 +108,27 @@ class Runner:
             sys.stderr.write(f"bench: graph capture unavailable ({type(e).__name__}: {e}); plain launches\n")
             graph = None
             torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        if graph is not None:
-            full, rest = divmod(steps, per_graph)
-            for _ in range(full):
-                graph.replay()
-            for i in range(rest):
-                launch_step(i % n_variants)
-        else:
-            for i in range(steps):
-                launch_step(i % n_variants)
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps, mode
+        times = []
+        for _ in range(self.REGIONS):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            if graph is not None:
+                full, rest = divmod(steps, per_graph)
+                for _ in range(full):
+                    graph.replay()
+                for i in range(rest):
+                    launch_step(i % n_variants)
+            else:
+                for i in range(steps):
+                    launch_step(i % n_variants)
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / steps)
+        times.sort()
+        if stats is not None:
+            stats.update(regions=len(times), ms_per_step_min=times[0], ms_per_step_max=times[-1])
+        return times[len(times) // 2], mode
 
 
 def bench_q8_gemv(r: Runner, O, M, steps, warmup, seed=0, copies=None):
@@ -137,7 +147,8 @@ def bench_q8_gemv(r: Runner, O, M, steps, warmup, seed=0, copies=None):
     xd, bd = r.upload(x), r.upload(bias)
     outs = [r.torch.empty(M * N * 2, dtype=r.torch.uint8, device="cuda:0") for _ in range(copies)]
     desc = r.ffi.make_desc(r.ffi.RT_Q8_0H, (N, K), r.ffi.RT_F16, (1, M, K), False, True, True, r.ffi.RT_F16, (N,))
-    ms, mode = r.time_steps(lambda i: r.enqueue(desc, ws[i], xd, bd, outs[i]), steps, warmup, copies)
+    stats = {}
+    ms, mode = r.time_steps(lambda i: r.enqueue(desc, ws[i], xd, bd, outs[i]), steps, warmup, copies, stats)
     # parity of what was just timed, against the oracle on the same inputs
     got = outs[(steps - 1) % copies].cpu().numpy().view(np.float16).reshape(1, M, N)
     ref = O.matmul_ref(wbuf, O.Q8_0H, (N, K), x, O.F16, x.shape, bias, False, True, True)
@@ -145,7 +156,7 @@ def bench_q8_gemv(r: Runner, O, M, steps, warmup, seed=0, copies=None):
     if not err <= 2e-2:
         raise RuntimeError(f"bench output differs from the oracle: max_rel_err={err}")
     return dict(ms=ms, bytes=per, gbps=per / (ms * 1e-3) / 1e9, mode=mode, copies=copies, err=err,
-                inputs=(wbuf, x, bias))
+                inputs=(wbuf, x, bias), stats=stats)
 
 
 def bench_q8_gemm(r: Runner, O, steps, warmup, act=0):
@@ -597,12 +608,12 @@ def main():
     if not args.no_secondary:
         sec_steps = max(200, args.steps // 4)
         warm = bench_q8_gemv(r, O, 1, sec_steps, max(20, args.warmup // 4), copies=1)
-        warm.pop("inputs")
+        warm.pop("inputs"), warm.pop("stats")
         secondary.append({"workload": "C2 Q8_0 GEMV M=1, warm: one weight copy, resident in the Infinity Cache (not HBM)",
                           "value": round(warm["gbps"], 1), "unit": "GB/s", "ms_per_step": warm["ms"]})
         for M in (4, 8):
             s = bench_q8_gemv(r, O, M, sec_steps, max(20, args.warmup // 4), seed=M)
-            s.pop("inputs")
+            s.pop("inputs"), s.pop("stats")
             secondary.append({"workload": f"C2 Q8_0 GEMV M={M}", "value": round(s["gbps"], 1), "unit": "GB/s",
                               "ms_per_step": s["ms"], "frac_hbm_peak": round(s["gbps"] / HBM_PEAK_GBPS, 4)})
         gsteps = max(50, args.steps // 40)
@@ -632,6 +643,10 @@ def main():
                         "Q8_0H W[10240x2560]^T + f16 bias, M=1",
             "weight_copies_rotated": head["copies"],
             "launch": head["mode"],
+            "timed_regions": head["stats"]["regions"],
+            "ms_per_step_is": "median over the timed regions of `steps` launches each",
+            "ms_per_step_min": head["stats"]["ms_per_step_min"],
+            "ms_per_step_max": head["stats"]["ms_per_step_max"],
             "max_rel_err_vs_oracle": head["err"],
         },
         "roofline": {
@@ -642,7 +657,7 @@ def main():
             "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4),
             "traffic": GEMV_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": head["bytes"],
-            "kernel": "gemv_q8h_mfma_kernel",
+            "kernel": "gemv_q8h_rowdot_kernel<5, 1, 1>",
         },
         "cpu_baseline": {
             "value": round(head["bytes"] / cpu_s / 1e9, 3),

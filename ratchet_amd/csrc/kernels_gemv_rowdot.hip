@@ -1,0 +1,260 @@
+// Row-streaming Q8_0H GEMV for one or two activation vectors (the decode step).
+//
+//   y[j, n] = sum_b d[n, b] * ( sum_{k in block b} q[n, k] * x[j, k] )  (+ bias)
+//
+// The weight matrix is read as what it is in memory, one long run of bytes: a half-wave
+// (32 lanes) owns one weight row and every load instruction fetches 512 consecutive bytes of
+// it, 16 per lane, so a wavefront touches whole 128-byte lines and touches each exactly
+// once.  That is what lets the loads be non-temporal (the stream is not kept in the
+// caches it passes through) and it is worth 0.8 us of 7.6 at the Phi-2 shape against
+// the matrix-core kernel, whose operand layout (16 rows x 64 bytes per instruction) reads
+// every line in two halves from two instructions.  Measured with that kernel's own
+// arithmetic on a linear address pattern: 7.56 -> 7.06 us, non-temporal 6.78 us; the
+// same non-temporal loads on the 16-row pattern: 9.05 us.
+//
+// A lane multiplies its 16 codes with the 16 activations at the same K positions:
+// the codes are widened to f16 exactly, v_dot2_f32_f16 accumulates the products in
+// f32 and the half-block's sum is scaled by the block's f16 scale in f32, so no weight is
+// rounded.  The 32 partial sums of a row meet in five DPP additions; nothing is
+// summed across wavefronts and the kernel ends without a barrier.  The activations
+// are staged once per workgroup in LDS (their loads are issued first and the one
+// barrier waits for them only), then held in registers.
+//
+// With more vectors the dot products repeat per vector while a matrix instruction takes
+// 16 vectors at once: this kernel wins for one and two vectors (6.4 / 7.2 us against
+// 7.6 / 7.8 us) and loses from three (9.0 against 8.6 us), where the matrix-core
+// kernel stays in charge.
+//
+// Roles in the reference: ops/gemv.rs:333-558 (subgroup GEMV), kernel_builder.rs:222-240
+// (unpack), dtype/blocks.rs:61-74 (segment layout).
+#include "device_common.h"
+
+namespace rt {
+
+struct GemvRowdotArgs {
+    const uint8_t *qs;
+    const half_t *scales;
+    const half_t *X;
+    const half_t *bias;
+    half_t *out;
+    int64_t M;              // weight rows
+    int64_t a_stack, b_stack;
+    int64_t b_bs, b_js;
+    int64_t o_bs, o_is, o_js;
+    int has_bias, bias_on_rows, act;
+};
+
+constexpr int kRowdotWaves = 4;
+
+// (q ^ 0x80) is q + 128 as an unsigned byte; 0x6400 | byte is the f16 1024 + byte; minus 1152 leaves q
+__device__ __forceinline__ void rowdot_cvt_i8x4(uint32_t v, half2_t &lo, half2_t &hi) {
+    v ^= 0x80808080u;
+    const half2_t off = {(half_t)1152.0f, (half_t)1152.0f};
+    lo = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u)) - off;
+    hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u)) - off;
+}
+
+template <int CTRL, int ROWMASK> __device__ __forceinline__ float rowdot_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true));
+}
+// Sum over each half-wave, valid in lanes 16..31 and 48..63; with WHOLE the sum over all 64 lanes, valid in lanes 48..63.
+template <bool WHOLE> __device__ __forceinline__ float rowdot_sum(float v) {
+    v += rowdot_dpp<0x128, 0xf>(v); // row_ror:8
+    v += rowdot_dpp<0x124, 0xf>(v); // row_ror:4
+    v += rowdot_dpp<0x122, 0xf>(v); // row_ror:2
+    v += rowdot_dpp<0x121, 0xf>(v); // row_ror:1: every lane of a row of 16 holds the row's sum
+    v += rowdot_dpp<0x142, 0xa>(v); // row_bcast:15: rows 1 and 3 add the row before them
+    if (WHOLE) v += rowdot_dpp<0x143, 0xc>(v); // row_bcast:31: rows 2 and 3 add lane 31
+    return v;
+}
+
+// K = 512 * STEPS * SEG.  SEG == 1: a wavefront owns two rows, one per half-wave.  SEG == 2: a
+// wavefront owns one row and each half-wave half of its K.  NCT activation vectors (1 or 2).
+// Offsets inside a workgroup's rows are 32-bit; the workgroup's base is 64-bit and wave-uniform.
+template <int STEPS, int SEG, int NCT>
+__global__ __launch_bounds__(kRowdotWaves * 64) void gemv_q8h_rowdot_kernel(GemvRowdotArgs g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int K = 512 * STEPS * SEG;
+    constexpr int KQ = K / 32;
+    constexpr int THREADS = kRowdotWaves * 64;
+    constexpr int ROWS = kRowdotWaves * 2 / SEG;      // rows per workgroup
+    half_t *xs = (half_t *)smem;                      // [NCT][K]
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int c = lane & 31, hr = lane >> 5;
+    const int64_t s = blockIdx.y;
+    const int64_t sa = g.a_stack == 1 ? 0 : s, sb = g.b_stack == 1 ? 0 : s;
+    const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+    const int rw = SEG == 1 ? 2 * wave + hr : wave;                 // this lane's row within the workgroup
+    const int last = (int)min((int64_t)(ROWS - 1), g.M - 1 - row0); // rows past the end repeat the last one; never stored
+    const uint32_t rc = (uint32_t)min(rw, last);
+    const uint32_t kbase = SEG == 1 ? 0u : (uint32_t)hr * (512u * STEPS);
+
+    // 1. the activations: the workgroup stages all of K per vector
+    constexpr int XV = (NCT * K / 8 + THREADS - 1) / THREADS;
+    uint4_t xv[XV];
+    const half_t *xg = g.X + sb * g.b_bs;
+#pragma unroll
+    for (int i = 0; i < XV; i++) {
+        const uint32_t v = min((uint32_t)(i * THREADS + t), (uint32_t)(NCT * K / 8 - 1)); // threads past the end re-read the last vector
+        const uint32_t j = v / (K / 8), kv = v % (K / 8);
+        xv[i] = *(const uint4_t *)(xg + (j * g.b_js + 8 * kv));
+    }
+    asm volatile("" ::: "memory"); // keep the loads in this order
+    // 2. the weight stream: 16 bytes per lane and step, 512 consecutive bytes per half-wave
+    const uint8_t *qp = g.qs + (sa * g.M + row0) * K + (rc * (uint32_t)K + kbase + 16u * c);
+    uint4_t w[STEPS];
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) w[st] = __builtin_nontemporal_load((const uint4_t *)(qp + 512 * st));
+    asm volatile("" ::: "memory");
+    // 3. the scale of this lane's half block at every step, then the epilogue's bias (unconditional: without
+    //    a bias it reads a scale and the value is dropped; a branch here would wait for every load above)
+    const half_t *sp = g.scales + (sa * g.M + row0) * KQ + (rc * (uint32_t)KQ + kbase / 32 + (c >> 1));
+    uint16_t dsc[STEPS];
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) dsc[st] = *(const uint16_t *)(sp + 16 * st);
+    uint16_t bias_raw[NCT];
+#pragma unroll
+    for (int j = 0; j < NCT; j++) {
+        const half_t *bp = g.has_bias ? g.bias + (g.bias_on_rows ? row0 + rc : (int64_t)j) : sp;
+        bias_raw[j] = *(const uint16_t *)bp;
+    }
+    asm volatile("" ::: "memory");
+    // 4. activations -> LDS; the barrier waits for the LDS writes, not for the weights
+#pragma unroll
+    for (int i = 0; i < XV; i++) {
+        const uint32_t v = i * THREADS + t;
+        if (v < NCT * K / 8) *(uint4_t *)(xs + 8 * v) = xv[i];
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // this lane's 16 activations per step; few enough to sit in registers while the weights are in flight
+    constexpr bool HOIST = NCT * STEPS <= 6;
+    uint4_t xa[HOIST ? NCT : 1][HOIST ? STEPS : 1], xb[HOIST ? NCT : 1][HOIST ? STEPS : 1];
+    const half_t *xl = xs + kbase + 16 * c;
+    if (HOIST) {
+#pragma unroll
+        for (int j = 0; j < NCT; j++)
+#pragma unroll
+            for (int st = 0; st < STEPS; st++) {
+                xa[j][st] = *(const uint4_t *)(xl + j * K + 512 * st);
+                xb[j][st] = *(const uint4_t *)(xl + j * K + 512 * st + 8);
+            }
+    }
+    // 5. dot products, one block scale per step
+    float acc[NCT];
+#pragma unroll
+    for (int j = 0; j < NCT; j++) acc[j] = 0.f;
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+        half2_t wh[8];
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t ww = w[st][d];
+            rowdot_cvt_i8x4(ww, wh[2 * d], wh[2 * d + 1]);
+        }
+        const float sc = (float)__builtin_bit_cast(half_t, dsc[st]);
+#pragma unroll
+        for (int j = 0; j < NCT; j++) {
+            uint4_t ya, yb;
+            if (HOIST) ya = xa[j][st], yb = xb[j][st];
+            else ya = *(const uint4_t *)(xl + j * K + 512 * st), yb = *(const uint4_t *)(xl + j * K + 512 * st + 8);
+            float p = 0.f;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t xw = ya[d];
+                p = __builtin_amdgcn_fdot2(wh[d], __builtin_bit_cast(half2_t, xw), p, false);
+            }
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t xw = yb[d];
+                p = __builtin_amdgcn_fdot2(wh[4 + d], __builtin_bit_cast(half2_t, xw), p, false);
+            }
+            acc[j] = fmaf(sc, p, acc[j]);
+        }
+    }
+    // 6. the row's lanes meet; one lane per row writes
+    const bool writer = SEG == 1 ? c == 16 : lane == 48;
+#pragma unroll
+    for (int j = 0; j < NCT; j++) {
+        const float v = rowdot_sum<SEG == 2>(acc[j]);
+        if (writer && rw <= last) {
+            const float b = g.has_bias ? (float)__builtin_bit_cast(half_t, bias_raw[j]) : 0.f;
+            g.out[s * g.o_bs + (row0 + rw) * g.o_is + j * g.o_js] = (half_t)rt_act(v + b, g.act);
+        }
+    }
+}
+
+// Tunable: 1 = never take this kernel (for comparisons).
+RT_TUNABLE(g_gemv_rowdot_disable, 0);
+
+template <int STEPS, int SEG, int NCT>
+static hipError_t launch_rowdot(dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
+    constexpr size_t lds = (size_t)NCT * 512 * STEPS * SEG * 2;
+    if constexpr (lds > 48 * 1024) {
+        const hipError_t e = ensure_lds_limit<&gemv_q8h_rowdot_kernel<STEPS, SEG, NCT>>();
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((gemv_q8h_rowdot_kernel<STEPS, SEG, NCT>), grid, dim3(kRowdotWaves * 64), lds, st, g);
+    return hipGetLastError();
+}
+
+template <int SEG, int NCT>
+static hipError_t launch_rowdot_steps(int steps, dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
+    if constexpr (SEG == 1) { // two half-waves per row only take over where one would need more than 10 steps
+        switch (steps) {
+        case 1: return launch_rowdot<1, SEG, NCT>(grid, st, g);
+        case 2: return launch_rowdot<2, SEG, NCT>(grid, st, g);
+        case 3: return launch_rowdot<3, SEG, NCT>(grid, st, g);
+        case 4: return launch_rowdot<4, SEG, NCT>(grid, st, g);
+        case 5: return launch_rowdot<5, SEG, NCT>(grid, st, g);
+        default: break;
+        }
+    }
+    switch (steps) {
+    case 6: return launch_rowdot<6, SEG, NCT>(grid, st, g);
+    case 7: return launch_rowdot<7, SEG, NCT>(grid, st, g);
+    case 8: return launch_rowdot<8, SEG, NCT>(grid, st, g);
+    case 9: return launch_rowdot<9, SEG, NCT>(grid, st, g);
+    case 10: return launch_rowdot<10, SEG, NCT>(grid, st, g);
+    default: return hipErrorNotSupported;
+    }
+}
+
+// Q8_0H weights, one or two f16 activation vectors, K a multiple of 512 up to 5120 or of 1024 up to 10240.
+// hipErrorNotSupported: the shape or alignment does not fit and another kernel must run.
+hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
+                                  hipStream_t stream, const DeviceInfo &dev) {
+    (void)dev;
+    if (g_gemv_rowdot_disable) return hipErrorNotSupported;
+    if (p.a_dt != RT_Q8_0H || p.act_dt != RT_F16 || p.N < 1 || p.N > 2 || p.K < 512 || p.K % 512 != 0)
+        return hipErrorNotSupported;
+    if (p.stacks > 65535 || p.b_ks != 1 || p.M < 1) return hipErrorNotSupported;
+    const int64_t bjs = p.N == 1 ? 0 : p.b_js;
+    if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (bjs * 2) % 16 || (p.b_bs * 2) % 16) return hipErrorNotSupported;
+    int seg = 1, steps = (int)(p.K / 512);
+    if (steps > 10) {
+        if (p.K % 1024 != 0 || p.K > 10240) return hipErrorNotSupported;
+        seg = 2, steps = (int)(p.K / 1024);
+    }
+    const int rows = kRowdotWaves * 2 / seg;
+    const int64_t groups = (p.M + rows - 1) / rows;
+    if (groups > 0x7fffffff) return hipErrorNotSupported;
+
+    GemvRowdotArgs g{};
+    const uint64_t numel = (uint64_t)p.a_stack * p.M * p.K;
+    g.qs = (const uint8_t *)A;
+    g.scales = (const half_t *)((const uint8_t *)A + rt_q8_0_scale_offset(numel));
+    g.X = (const half_t *)B, g.bias = (const half_t *)bias, g.out = (half_t *)out;
+    g.M = p.M;
+    g.a_stack = p.a_stack, g.b_stack = p.b_stack;
+    g.b_bs = p.b_bs, g.b_js = bjs;
+    g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
+    g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
+    dim3 grid((unsigned)groups, (unsigned)p.stacks);
+    if (seg == 1) return p.N == 1 ? launch_rowdot_steps<1, 1>(steps, grid, stream, g) : launch_rowdot_steps<1, 2>(steps, grid, stream, g);
+    return p.N == 1 ? launch_rowdot_steps<2, 1>(steps, grid, stream, g) : launch_rowdot_steps<2, 2>(steps, grid, stream, g);
+}
+
+} // namespace rt

@@ -201,6 +201,52 @@ def test_q8_streaming_regular_and_ragged_variants(device, oracle):
     assert np.array_equal(got, dq[:, cols].T.astype(adt))
 
 
+def test_q8_row_streaming_one_and_two_vectors(device, oracle):
+    """Q8_0H weights against one or two vectors with K a multiple of 512 take the row-streaming kernel: every
+    step count of the one-row-per-half-wave form (K = 512 .. 5120), the two-half-waves-per-row form
+    (K = 6144 .. 10240 in steps of 1024), row counts off the 8 (4) rows of a workgroup, stacks of weights and of
+    activations with broadcast either way, the bias along the rows (trans_out) and along the vectors, and a
+    fused activation; then one-hot activations, bit for bit, with -128 planted."""
+    dt = DType.Q8_0H
+    cases = [(1, 1, 64, 512 * k) for k in range(1, 11)] + [(1, 1, 40, 1024 * k) for k in range(6, 11)]
+    cases += [(1, 2, 61, 2560), (1, 2, 3, 1024), (1, 1, 1, 512), (1, 2, 27, 8192), (1, 1, 10240, 2560), (1, 2, 13, 10240),
+              (3, 1, 19, 1536), (2, 2, 9, 7168)]
+    for i, (S, M, N, K) in enumerate(cases):
+        rng = np.random.default_rng(260 + i)
+        for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
+            w = (rng.standard_normal((ws, N, K)) * 0.05).astype(np.float32)
+            buf = oracle.make_q8_0h(w)
+            x = rng.standard_normal((xs_, M, K)).astype(np.float16)
+            for to in (True, False):
+                bias = rng.standard_normal(N if to else M).astype(np.float16) if (i + to) % 3 else None
+                got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (ws, N, K)), Tensor.from_data(x),
+                                 None if bias is None else Tensor.from_data(bias), False, True, to)
+                want = oracle.matmul_ref(buf, oracle.Q8_0H, (ws, N, K), x, oracle.F16, x.shape, bias, False, True, to)
+                check(oracle, got, want, DType.F16, (S, ws, xs_, M, N, K, to))
+    # GELU / SiLU behind the Linear, fused
+    rng = np.random.default_rng(280)
+    N, K = 100, 3072
+    buf = oracle.make_q8_0h((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    x = rng.standard_normal((1, 2, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    for name, act in (("gelu", oracle.ACT_GELU), ("silu", oracle.ACT_SILU)):
+        y = getattr(Tensor.from_quantized(buf, dt, (N, K)).to(device).gemm(
+            Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device), False, True, True), name)().resolve()
+        want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, bias, False, True, True, act=act)
+        assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
+    # one-hot: the dequantized weight, bit for bit, in both forms
+    for N, K in ((37, 2560), (21, 10240)):
+        buf = q8_weight(oracle, rng, N, K, dt)
+        buf[: N * K][5::97] = 0x80
+        dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
+        for M in (1, 2):
+            cols = np.concatenate([[5 + 97 * 3], rng.integers(0, K, size=M)])[:M]
+            x = np.zeros((M, K), dtype=np.float16)
+            x[np.arange(M), cols] = 1
+            got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (N, K)), Tensor.from_data(x), None, False, True, True)
+            assert np.array_equal(got, dq[:, cols].T.astype(np.float16)), (N, K, M)
+
+
 @pytest.mark.parametrize("dt", [DType.Q8_0H, DType.Q8_0F], ids=["q8_0h", "q8_0f"])
 def test_q8_one_hot_is_bit_exact_dequant(device, oracle, dt):
     """A one-hot activation selects one dequantized weight per row: the GEMV / GEMM
