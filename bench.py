@@ -182,9 +182,11 @@ def bench_q8_gemm(r: Runner, O, steps, warmup, act=0):
                 tflops=flops / (ms * 1e-3) / 1e12, mode=mode)
 
 
-def bench_f16_gemm(r: Runner, O, steps, warmup):
-    """The C4 shape with plain f16 weights: X [512 x 2560] . W[10240 x 2560]^T + bias (the f16 GEMM headline)."""
-    M, N, K = 512, 10240, 2560
+def bench_f16_gemm(r: Runner, O, steps, warmup, M=512):
+    """The C4 shape with plain f16 weights: X [512 x 2560] . W[10240 x 2560]^T + bias (the f16 GEMM headline).
+    Larger M (more activation rows against the same weight) shows what the kernel does when the shape is not
+    the limit: at 512 rows the grid is exactly one workgroup per compute unit."""
+    N, K = 10240, 2560
     rng = np.random.default_rng(5)
     w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
     x = rng.standard_normal((1, M, K)).astype(np.float16)
@@ -198,8 +200,9 @@ def bench_f16_gemm(r: Runner, O, steps, warmup):
     err = O.max_rel_err(got, ref)
     if not err <= 2e-2:
         raise RuntimeError(f"f16 GEMM output differs from float64: max_rel_err={err}")
-    return dict(workload="C4 shape, f16 weights: X[512x2560] f16 . W[10240x2560]^T f16 + bias", ms=ms,
-                tflops=2.0 * M * N * K / (ms * 1e-3) / 1e12, mode=mode)
+    return dict(workload=f"C4 shape, f16 weights: X[{M}x2560] f16 . W[10240x2560]^T f16 + bias", ms=ms,
+                tflops=2.0 * M * N * K / (ms * 1e-3) / 1e12, mode=mode, flops=2.0 * M * N * K,
+                bytes=2 * (M * K + N * K + N + M * N))
 
 
 def bench_generic(r: Runner, O, name, lhs, lhs_dt, lhs_shape, rhs, rhs_shape, bias, flags, act, flops, nbytes, steps,
@@ -592,8 +595,10 @@ def main():
     from oracle import oracle as O
     r = Runner()
     if args.gemm_only:
-        for g in (bench_f16_gemm(r, O, 100, 10), bench_q8_gemm(r, O, 100, 10)):
-            print(json.dumps({"workload": g["workload"], "tflops": round(g["tflops"], 1), "ms_per_step": g["ms"]}))
+        for g in (bench_f16_gemm(r, O, 100, 10), bench_q8_gemm(r, O, 100, 10), bench_f16_gemm(r, O, 50, 5, M=2048),
+                  bench_f16_gemm(r, O, 50, 5, M=4096)):
+            print(json.dumps({"workload": g["workload"], "tflops": round(g["tflops"], 1), "ms_per_step": g["ms"],
+                              "frac_mfma_f16_peak": round(g["tflops"] / MFMA_F16_PEAK_TFLOPS, 4)}))
         return 0
 
     if args.q4k_only:

@@ -23,6 +23,26 @@ def test_header_symbols_are_exported():
     assert sorted(_ffi.SIGNATURES) == syms  # the Python binding covers the same set
 
 
+def test_rust_crate_declares_every_symbol():
+    """crates/ratchet-hip-sys/src/lib.rs (source only: no rustc in the image) declares every symbol the header
+    exports, with as many arguments, and nothing the header does not have."""
+    text = open(os.path.join(ROOT, "include", "ratchet_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    header = {m.group(1): m.group(2) for m in re.finditer(r"RT_API[^;(]*?\b(rt_[a-z0-9_]+)\s*\(([^;]*?)\)\s*;", text, flags=re.S)}
+    rs = open(os.path.join(ROOT, "crates", "ratchet-hip-sys", "src", "lib.rs")).read()
+    rs = re.sub(r"//[^\n]*", "", rs)
+    rust = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (rt_[a-z0-9_]+)\s*\(([^;]*?)\)\s*(?:->[^;]*)?;", rs, flags=re.S)}
+    assert sorted(rust) == sorted(header) == header_symbols()
+    nargs = lambda a: 0 if a.strip() in ("", "void") else a.count(",") + 1
+    for name in header:
+        assert nargs(rust[name]) == nargs(header[name]), name
+    # the structs the entry points take exist with the header's field counts
+    for struct, fields in (("rt_matmul_desc", 13), ("rt_gemm_spec", 13), ("rt_attention_desc", 14),
+                           ("rt_gguf_tensor_info", 6), ("rt_gguf_value", 7)):
+        body = re.search(r"pub struct %s \{(.*?)\n\}" % struct, rs, flags=re.S).group(1)
+        assert len(re.findall(r"pub \w+:", body)) == fields, struct
+
+
 def test_status_and_kernel_strings():
     L = _ffi.lib()
     assert L.rt_status_string(_ffi.RT_OK) == b"RT_OK"
