@@ -538,6 +538,47 @@ def bench_q4k(r: Runner, O, rows, steps):
     return out
 
 
+def read_calibration(r: Runner, O, steps, warmup):
+    """Context for the headline: on the same 20 rotated copies of the 27.85 MB weight and with the same graph
+    timing, what a launch costs that does nothing, what one costs that only reads the buffer (consecutive
+    addresses, with and without non-temporal loads; and in the 16-row pattern the matrix-core kernel reads it
+    in), and the GEMV itself.  The probes are in ratchet_amd/libratchet_probes.so (csrc/bench_probes.hip)."""
+    N, K = 10240, 2560
+    rng = np.random.default_rng(0)
+    wbuf = O.make_q8_0h((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    copies = max(2, -(-2 * INFINITY_CACHE_BYTES // wbuf.size))
+    ws = [r.upload(wbuf) for _ in range(copies)]
+    sink = r.torch.zeros(4096, dtype=r.torch.uint8, device="cuda:0")
+    P = ctypes.CDLL(os.path.join(ROOT, "ratchet_amd", "libratchet_probes.so"))
+    vp, u64, i64 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int64
+    P.probe_empty.argtypes, P.probe_read_linear.argtypes = [vp, vp], [vp, u64, ctypes.c_int, vp, vp]
+    P.probe_read_rows16.argtypes = [vp, i64, i64, vp, vp]
+    stream = lambda: vp(r.torch.cuda.current_stream().cuda_stream)
+    nbytes = wbuf.size - wbuf.size % 16
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(f"probe launch failed: hipError {rc}")
+
+    x = rng.standard_normal((1, 1, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    xd, bd = r.upload(x), r.upload(bias)
+    out = r.torch.empty(N * 2, dtype=r.torch.uint8, device="cuda:0")
+    desc = r.ffi.make_desc(r.ffi.RT_Q8_0H, (N, K), r.ffi.RT_F16, (1, 1, K), False, True, True, r.ffi.RT_F16, (N,))
+    rows = []
+    for name, step, nb in (
+            ("empty kernel (one wavefront)", lambda i: ok(P.probe_empty(vp(sink.data_ptr()), stream())), 0),
+            ("read only, consecutive addresses", lambda i: ok(P.probe_read_linear(vp(ws[i].data_ptr()), nbytes, 0, vp(sink.data_ptr()), stream())), nbytes),
+            ("read only, consecutive addresses, non-temporal loads", lambda i: ok(P.probe_read_linear(vp(ws[i].data_ptr()), nbytes, 1, vp(sink.data_ptr()), stream())), nbytes),
+            ("read only, 16 rows x 64 bytes per load (the int8 codes alone)", lambda i: ok(P.probe_read_rows16(vp(ws[i].data_ptr()), N, K, vp(sink.data_ptr()), stream())), N * K),
+            ("Q8_0H GEMV M=1 (the headline)", lambda i: r.enqueue(desc, ws[i], xd, bd, out), gemv_bytes(1, N, K))):
+        stats = {}
+        ms, mode = r.time_steps(step, steps, warmup, copies, stats)
+        rows.append({"launch": name, "us_per_launch": round(ms * 1e3, 3), "us_min": round(stats["ms_per_step_min"] * 1e3, 3),
+                     "bytes": nb, "GB/s": round(nb / (ms * 1e-3) / 1e9, 1) if nb else None, "timing": mode})
+    return {"read_calibration": rows, "weight_copies_rotated": copies, "steps": steps, "regions": Runner.REGIONS}
+
+
 def cpu_baseline(O, wbuf, x, bias, budget_s=1.5):
     """The oracle's reference path on the host cores, same inputs: median of >= 3 runs.  Returns
     (seconds, runs) for the whole path (dequantize W to f32, f32 GEMV, bias, cast) and the same for the
@@ -571,6 +612,8 @@ def main():
                     help="run only the two C4 GEMM workloads (f16 and Q8_0H weights) and print their lines; for profiling")
     ap.add_argument("--q4k-only", action="store_true",
                     help="run only the Q4_K prefill workload (C5 at 256 rows) and print its line; for profiling")
+    ap.add_argument("--read-calibration", action="store_true",
+                    help="only time an empty launch and read-only passes over the rotated weight copies next to the GEMV")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 20 device-to-device copies of 256 MiB (reference dispatches for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -594,6 +637,9 @@ def main():
         return 0
     from oracle import oracle as O
     r = Runner()
+    if args.read_calibration:
+        print(json.dumps(read_calibration(r, O, min(args.steps, 2000), min(args.warmup, 100))))
+        return 0
     if args.gemm_only:
         for g in (bench_f16_gemm(r, O, 100, 10), bench_q8_gemm(r, O, 100, 10), bench_f16_gemm(r, O, 50, 5, M=2048),
                   bench_f16_gemm(r, O, 50, 5, M=4096)):

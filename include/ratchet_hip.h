@@ -52,7 +52,10 @@ typedef enum rt_status {
     RT_ERR_INVALID_SHAPE = 2,  /* broadcast failure, ka != kb, bias not a vector / wrong length, */
                                /* rank < 2 at execution, operand stacks neither equal nor 1      */
     RT_ERR_DTYPE_MISMATCH = 3, /* (lhs, rhs) pair not allowed, or bias dtype != activation dtype */
-    RT_ERR_UNSUPPORTED = 4,    /* transposed quantized operand, K not a multiple of the block    */
+    RT_ERR_UNSUPPORTED = 4,    /* transposed quantized operand, K not a multiple of the block;   */
+                               /* at enqueue: a shape no kernel takes (more than 65535 stacks or */
+                               /* 65535 x 64 rows on the generic kernel's path, or a quantized   */
+                               /* operand that is not 16-byte aligned)                           */
     RT_ERR_NO_DEVICE = 5,      /* no HIP device / ordinal out of range                           */
     RT_ERR_HIP = 6,            /* a HIP runtime call failed; see rt_last_hip_error               */
     RT_ERR_OOM = 7             /* hipMalloc failed                                               */

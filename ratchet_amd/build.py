@@ -17,6 +17,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "_build")
 LIB = os.path.join(HERE, "libratchet_hip.so")
+# measurement probes of bench.py --read-calibration: their own library, not part of the product
+PROBES_SRC = "bench_probes.hip"
+PROBES_LIB = os.path.join(HERE, "libratchet_probes.so")
 ARCH = "gfx950"
 
 SOURCES = ["api.cpp", "spec.cpp", "gguf.cpp", "kernels_blocks.hip", "kernels_softmax.hip", "kernels_unary.hip", "kernels_attention.hip", "kernels_gemv.hip", "kernels_gemv_mfma.hip", "kernels_gemv_rowdot.hip",
@@ -74,6 +77,12 @@ def build(force: bool = False, verbose: bool = True) -> str:
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"link failed:\n{res.stderr}")
+    probes_src = os.path.join(CSRC, PROBES_SRC)
+    if force or _stale(PROBES_LIB, [probes_src, os.path.abspath(__file__)]):
+        cmd = [hipcc(), *FLAGS, "-shared", probes_src, "-o", PROBES_LIB]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {PROBES_SRC}:\n{res.stderr}")
     if verbose:
         print(f"built {LIB}")
     return LIB

@@ -193,6 +193,7 @@ rt_status rt_buf_alloc(rt_ctx *ctx, uint64_t nbytes, void **dptr) {
     if (!ctx || !dptr) return RT_ERR_INVALID_ARG;
     DeviceGuard dg(ctx->dev.ordinal);
     *dptr = nullptr;
+    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
     hipError_t e = hipMalloc(dptr, nbytes ? nbytes : 4);
     if (e != hipSuccess) return hip_fail(ctx, "hipMalloc", e);
     return RT_OK;
@@ -202,6 +203,7 @@ rt_status rt_buf_free(rt_ctx *ctx, void *dptr) {
     if (!ctx) return RT_ERR_INVALID_ARG;
     if (!dptr) return RT_OK;
     DeviceGuard dg(ctx->dev.ordinal);
+    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
     hipError_t e = hipFree(dptr);
     if (e != hipSuccess) return hip_fail(ctx, "hipFree", e);
     return RT_OK;
@@ -211,6 +213,7 @@ rt_status rt_buf_upload(rt_ctx *ctx, void *dst_dev, const void *src_host, uint64
     if (!ctx || (nbytes && (!dst_dev || !src_host))) return RT_ERR_INVALID_ARG;
     if (!nbytes) return RT_OK;
     DeviceGuard dg(ctx->dev.ordinal);
+    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
     hipError_t e = hipMemcpyAsync(dst_dev, src_host, nbytes, hipMemcpyHostToDevice, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(ctx, "hipMemcpyAsync(H2D)", e);
     return RT_OK;
@@ -220,6 +223,7 @@ rt_status rt_buf_download(rt_ctx *ctx, void *dst_host, const void *src_dev, uint
     if (!ctx || (nbytes && (!dst_host || !src_dev))) return RT_ERR_INVALID_ARG;
     if (!nbytes) return RT_OK;
     DeviceGuard dg(ctx->dev.ordinal);
+    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
     hipError_t e = hipMemcpyAsync(dst_host, src_dev, nbytes, hipMemcpyDeviceToHost, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(ctx, "hipMemcpyAsync(D2H)", e);
     return RT_OK;
@@ -228,6 +232,7 @@ rt_status rt_buf_download(rt_ctx *ctx, void *dst_host, const void *src_dev, uint
 rt_status rt_sync(rt_ctx *ctx, void *stream) {
     if (!ctx) return RT_ERR_INVALID_ARG;
     DeviceGuard dg(ctx->dev.ordinal);
+    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
     hipError_t e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(ctx, "hipStreamSynchronize", e);
     return RT_OK;
@@ -301,6 +306,11 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
         if (e == hipErrorNotSupported)
             e = rt::launch_gemm(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
     }
+    // no kernel takes the shape (more than 65535 stacks or row tiles of the generic kernel, a misaligned
+    // quantized operand): a limit of this library, not a failure of the runtime
+    if (e == hipErrorNotSupported)
+        return fail(ctx, RT_ERR_UNSUPPORTED, "matmul: no kernel takes this shape (over 65535 stacks or 65535 row tiles, or a "
+                                             "quantized operand that is not 16-byte aligned)");
     if (e != hipSuccess) return hip_fail(ctx, "matmul launch", e);
     return RT_OK;
     RT_GUARD_END(ctx)

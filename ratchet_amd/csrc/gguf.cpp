@@ -4,7 +4,11 @@
 // Follows crates/ratchet-loader/src/gguf/gguf.rs:408-479 (Header::read), :164-180
 // (read_string), :330-377 (Value::read), :63-106 (TensorInfo) and :118-142
 // (ratchet_from_gguf); type tables from crates/ratchet-loader/src/lib.rs:62-140.
+// RT_HOST_ONLY leaves out the one function that talks to the device, so that the parser can be built
+// by a host compiler alone (the sanitizer build of the test suite does).
+#ifndef RT_HOST_ONLY
 #include <hip/hip_runtime.h>
+#endif
 
 #include <cstring>
 #include <stdexcept>
@@ -12,7 +16,9 @@
 #include <unordered_map>
 #include <vector>
 
+#ifndef RT_HOST_ONLY
 #include "device_common.h"
+#endif
 #include "spec.h"
 
 namespace {
@@ -303,10 +309,10 @@ rt_status rt_gguf_metadata_array_get(const rt_gguf *g, const char *key, uint64_t
 
 namespace rt {
 
-// Host image -> device tensor in this library's layout.  Returns a message on failure.
-rt_status gguf_load_tensor(const rt_gguf *g, const void *image, uint64_t size, uint64_t index, int32_t dst_dtype,
-                           void *staging, void *dst, hipStream_t stream, std::string &why, hipError_t &herr) {
-    herr = hipSuccess;
+// TensorInfo::byte_range (gguf.rs:100-105) against an image of `size` bytes: where tensor `index` begins, or why
+// it cannot lie in the image.  Offsets and sizes come from the file and are not trusted: neither sum may wrap.
+rt_status gguf_tensor_range(const rt_gguf *g, uint64_t size, uint64_t index, uint64_t *begin, uint64_t *numel_out,
+                            std::string &why) {
     if (index >= g->tensors.size()) return why = "tensor index out of range", RT_ERR_INVALID_ARG;
     const TensorInfo &ti = g->tensors[index];
     uint64_t numel = 1;
@@ -315,8 +321,23 @@ rt_status gguf_load_tensor(const rt_gguf *g, const void *image, uint64_t size, u
     if (numel % bn != 0) // gguf.rs:72-76
         return why = "the number of elements " + std::to_string(numel) + " is not divisible by the block size " + std::to_string(bn),
                RT_ERR_INVALID_SHAPE;
-    const uint64_t begin = g->tensor_data_offset + ti.offset;
-    if (begin > size || ti.size_in_bytes > size - begin) return why = "tensor data lies outside the image", RT_ERR_INVALID_ARG;
+    if (g->tensor_data_offset > size || ti.offset > size - g->tensor_data_offset)
+        return why = "tensor data lies outside the image", RT_ERR_INVALID_ARG;
+    const uint64_t b = g->tensor_data_offset + ti.offset;
+    if (ti.size_in_bytes > size - b) return why = "tensor data lies outside the image", RT_ERR_INVALID_ARG;
+    *begin = b, *numel_out = numel;
+    return RT_OK;
+}
+
+#ifndef RT_HOST_ONLY
+// Host image -> device tensor in this library's layout.  Returns a message on failure.
+rt_status gguf_load_tensor(const rt_gguf *g, const void *image, uint64_t size, uint64_t index, int32_t dst_dtype,
+                           void *staging, void *dst, hipStream_t stream, std::string &why, hipError_t &herr) {
+    herr = hipSuccess;
+    uint64_t begin = 0, numel = 0;
+    const rt_status rs = gguf_tensor_range(g, size, index, &begin, &numel, why);
+    if (rs != RT_OK) return rs;
+    const TensorInfo &ti = g->tensors[index];
     const uint8_t *src = (const uint8_t *)image + begin;
     if (numel == 0) return RT_OK;
     if (!dst) return why = "null destination", RT_ERR_INVALID_ARG;
@@ -337,5 +358,6 @@ rt_status gguf_load_tensor(const rt_gguf *g, const void *image, uint64_t size, u
     return why = "unsupported ggml dtype " + std::to_string(ti.ggml_dtype) + " for destination dtype " + std::to_string(dst_dtype), // gguf.rs:140
            RT_ERR_UNSUPPORTED;
 }
+#endif
 
 } // namespace rt

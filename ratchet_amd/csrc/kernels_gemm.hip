@@ -485,14 +485,14 @@ RT_TUNABLE(g_gemm_tile, 0);
 
 hipError_t launch_gemm(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                        hipStream_t stream, const DeviceInfo &dev) {
-    if (p.stacks > 65535) return hipErrorInvalidValue;
+    if (p.stacks > 65535) return hipErrorNotSupported;
     // 128 x 128 tiles unless they would leave the chip under two workgroups per compute unit
     int ts = 128;
     const int64_t big = ((p.M + 127) / 128) * ((p.N + 127) / 128) * p.stacks;
     if (big < 2 * (int64_t)dev.num_cus) ts = 64;
     if (g_gemm_tile == 64 || g_gemm_tile == 128) ts = g_gemm_tile;
     const int64_t gy = (p.M + ts - 1) / ts, gx = (p.N + ts - 1) / ts;
-    if (gy > 65535) return hipErrorInvalidValue;
+    if (gy > 65535) return hipErrorNotSupported;
     GemmArgs g{};
     g.A = A, g.B = B, g.bias = bias, g.out = out;
     g.M = p.M, g.N = p.N, g.K = p.K;
@@ -505,11 +505,11 @@ hipError_t launch_gemm(const Problem &p, const void *A, const void *B, const voi
 
     int amode;
     if (p.a_dt == RT_Q8_0F || p.a_dt == RT_Q8_0H) {
-        if (!aligned16(A)) return hipErrorInvalidValue;
+        if (!aligned16(A)) return hipErrorNotSupported;
         amode = LM_Q8;
         g.scales = (const uint8_t *)A + rt_q8_0_scale_offset((uint64_t)p.a_stack * p.M * p.K);
     } else if (p.a_dt == RT_Q4_K) {
-        if (!aligned16(A)) return hipErrorInvalidValue;
+        if (!aligned16(A)) return hipErrorNotSupported;
         amode = LM_Q4K;
     } else {
         amode = float_mode(A, esz, p.M, p.K, p.a_rs, p.a_ks, p.a_bs);

@@ -74,6 +74,17 @@ rt_status compute_c_shape(const Shape &a_in, const Shape &b_in, bool trans_lhs, 
     return RT_OK;
 }
 
+// The product of the extents stays below 2^56 (no intermediate overflows: every extent is at most 2^40).
+static bool numel_fits(const Shape &s) {
+    int64_t n = 1;
+    for (int64_t v : s) {
+        if (v == 0) return true;
+        if (n > (int64_t(1) << 56) / v) return false;
+        n *= v;
+    }
+    return true;
+}
+
 static rt_status read_desc(const rt_matmul_desc &d, Shape &a, Shape &b, Shape &bias, std::string *why) {
     if (!valid_dtype(d.lhs_dt) || !valid_dtype(d.rhs_dt) || (d.has_bias && !valid_dtype(d.bias_dt))) {
         set_why(why, "unknown dtype id");
@@ -94,6 +105,12 @@ static rt_status read_desc(const rt_matmul_desc &d, Shape &a, Shape &b, Shape &b
                 set_why(why, "dimension out of range");
                 return RT_ERR_INVALID_ARG;
             }
+    // element counts (and every offset derived from them) must stay far inside int64
+    for (const Shape *s : {&a, &b})
+        if (!numel_fits(*s)) {
+            set_why(why, "tensor of more than 2^56 elements");
+            return RT_ERR_INVALID_ARG;
+        }
     return RT_OK;
 }
 
@@ -124,6 +141,10 @@ rt_status validate(const rt_matmul_desc &d, std::string *why) {
     // OpGuards::check_shapes (ops/matmul.rs:442-451)
     st = compute_c_shape(a, b, d.trans_lhs, d.trans_rhs, d.trans_out, c, why);
     if (st != RT_OK) return st;
+    if (!numel_fits(c)) {
+        set_why(why, "output of more than 2^56 elements");
+        return RT_ERR_INVALID_ARG;
+    }
     // OpGuards::check_dtypes (ops/matmul.rs:453-478)
     if (!pair_allowed(d.lhs_dt, d.rhs_dt)) {
         set_why(why, "Failed to validate DTypes: lhs " + std::to_string(d.lhs_dt) + ", rhs " +

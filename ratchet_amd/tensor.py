@@ -253,6 +253,9 @@ class Attention:
             raise OperationError(_ffi.RT_ERR_INVALID_SHAPE, f"attention: kv_len {self.kv_len} of a cache of {cap}")
         if mask is not None and tuple(mask.shape[-2:]) != (Lq, self.kv_len):
             raise OperationError(_ffi.RT_ERR_INVALID_SHAPE, f"attention: mask {mask.shape} for [{Lq}, {self.kv_len}] scores")
+        if mask is not None and int(np.prod(mask.shape[:-2], dtype=np.int64)) != 1:
+            # the kernel applies ONE [q_len, kv_len] mask to every batch and head (rt_attention_desc has a row stride only)
+            raise OperationError(_ffi.RT_ERR_UNSUPPORTED, f"attention: a mask per batch or head ({mask.shape}) is not supported")
         d = _ffi.AttentionDesc()
         d.dtype, d.batch, d.heads, d.q_len, d.kv_len, d.head_dim = int(q.dt), B, H, Lq, self.kv_len, D
         d.q_strides[:] = [Lq * H * D, D, H * D] if q_rows_interleaved else [H * Lq * D, Lq * D, D]
@@ -324,6 +327,10 @@ class Tensor:
     def __init__(self, shape: Sequence[int], dt: DType, device: Device, storage=None, op: Optional[Matmul] = None):
         self.shape = tuple(int(s) for s in shape)
         self.dt, self.device, self.storage, self.op = DType(dt), device, storage, op
+        self.consumers = 0   # operator nodes built on this tensor
+        if op is not None:
+            for src in op.srcs():
+                src.consumers += 1
 
     # -- construction -------------------------------------------------------
     @staticmethod
@@ -471,7 +478,10 @@ class Tensor:
             return
         op, dev, torch = self.op, self.device, _torch()
         act = _ffi.RT_ACT_NONE
-        if isinstance(op, Unary) and FUSE_ACTIVATIONS and isinstance(op.input.op, Matmul) and not op.input.resolved():
+        # an activation behind a product nobody else reads runs in that product's epilogue; a product with a second
+        # consumer is computed once, rounded, and the activation reads it (as the reference's two operators do)
+        if (isinstance(op, Unary) and FUSE_ACTIVATIONS and isinstance(op.input.op, Matmul) and not op.input.resolved()
+                and op.input.consumers <= 1):
             act, op = op.act, op.input.op
         for src in op.srcs():
             src._execute()

@@ -113,6 +113,13 @@ def test_guards_without_a_device():
         q.attention(Tensor.from_data(np.zeros((1, 3, 4, 16), np.float16)), Tensor.from_data(np.zeros((1, 3, 4, 16), np.float16)))
     with pytest.raises(OperationError):
         q.attention(q, q, kv_len=5)
+    # one [q_len, kv_len] mask serves every batch and head; a mask per batch or head is refused, not misapplied
+    m = np.zeros((4, 4), np.float32)
+    q.attention(q, q, Tensor.from_data(m))
+    q.attention(q, q, Tensor.from_data(m.reshape(1, 1, 4, 4)))
+    for shape in ((2, 4, 4), (1, 2, 4, 4)):
+        with pytest.raises(OperationError, match="per batch or head"):
+            q.attention(q, q, Tensor.from_data(np.zeros(shape, np.float32)))
     with pytest.raises(InvariantError):
         Tensor.from_data(np.zeros((1, 2, 4, 16), np.float32)).attention(q, q)
 

@@ -419,6 +419,11 @@ def test_enqueue_errors(device):
     assert b"null" in L.rt_last_error(device.ctx)
     d = _ffi.make_desc(_ffi.RT_F32, (4, 8), _ffi.RT_F32, (9, 3))
     assert L.rt_matmul_enqueue(device.ctx, ctypes.byref(d), None, None, None, None, None) == _ffi.RT_ERR_INVALID_SHAPE
+    # more stacks than any kernel's grid takes: a limit of the library (UNSUPPORTED), not a runtime failure
+    d = _ffi.make_desc(_ffi.RT_F32, (70000, 2, 3), _ffi.RT_F32, (70000, 3, 2))
+    buf = torch.zeros(70000 * 6 * 4, dtype=torch.uint8, device="cuda")
+    st = L.rt_matmul_enqueue(device.ctx, ctypes.byref(d), buf.data_ptr(), buf.data_ptr(), None, ctypes.c_void_p(buf.data_ptr()), None)
+    assert st == _ffi.RT_ERR_UNSUPPORTED and L.rt_last_hip_error(device.ctx) == 0 or st == _ffi.RT_OK
     a = Tensor.from_data(np.zeros(8, np.float32)).to(device)
     b = Tensor.from_data(np.zeros((8, 3), np.float32)).to(device)
     with pytest.raises(OperationError):   # GEMMSpec::new: inputs must be at least 2D

@@ -283,6 +283,18 @@ def test_fused_equals_two_operators_for_f32(device, oracle):
         finally:
             rt_tensor.FUSE_ACTIVATIONS = True
         assert np.array_equal(fused, two), name
+    # a product with a second consumer is computed once and the activation reads it: both consumers see the same values
+    a16, b16 = a.astype(np.float16), b.astype(np.float16)
+    A16, B16 = Tensor.from_data(a16).to(device), Tensor.from_data(b16).to(device)
+    node = A16.matmul(B16, False, False)
+    act, again = node.gelu(), node.silu()
+    got = act.resolve().to(Device.CPU).storage
+    assert node.resolved()                            # not fused: the rounded product exists
+    prod16 = node.to(Device.CPU).storage
+    assert np.array_equal(got, oracle.unary(prod16, oracle.ACT_GELU).astype(np.float16)) or np.allclose(
+        got.astype(np.float32), oracle.unary(prod16, oracle.ACT_GELU).astype(np.float32), rtol=2e-3, atol=1e-6)
+    assert np.allclose(again.resolve().to(Device.CPU).storage.astype(np.float32),
+                       oracle.unary(prod16, oracle.ACT_SILU).astype(np.float32), rtol=2e-3, atol=1e-6)
     # an activation on a resolved product runs as its own operator
     prod = A.gemm(B_, Bi, False, False, False).resolve()
     np.testing.assert_array_equal(prod.gelu().resolve().to(Device.CPU).storage,
