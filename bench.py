@@ -40,7 +40,7 @@ INFINITY_CACHE_BYTES = 256 << 20
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy); the commands and
 # readings are in profiles/gemv_q8_phi2_m1_pmc.txt.  A counter reading cannot be taken inside
 # this script, so the figure is the recorded one for the M=1 workload.
-GEMV_TRAFFIC_BYTES = 28041933
+GEMV_TRAFFIC_BYTES = 28149248
 
 
 def gemv_bytes(M, N, K):
