@@ -505,6 +505,11 @@ def other_configs(r: Runner, O):
                              (False, True, False), np.float16, 1342177280, 22020096, 200, 2e-2))
     out.append(bench_generic(r, O, "C3 PV f16 [32x512x512].[32x512x80]", p, ffi.RT_F16, p.shape, v, v.shape, None,
                              (False, False, False), np.float16, 1342177280, 22020096, 200, 2e-2))
+    # the phi2 / whisper spelling of the score product: f32 operands, the key permuted beforehand, matmul(false, false)
+    # (crates/ratchet-models/src/phi2/attn.rs:139-142): reads 2 x 5.2 MB, writes 33.6 MB of f32 scores
+    qf, ktf = q.astype(np.float32), np.ascontiguousarray(k.astype(np.float32).transpose(0, 1, 3, 2))
+    out.append(bench_generic(r, O, "C3 QK^T f32, key permuted beforehand [32x512x80].[32x80x512]", qf, ffi.RT_F32, qf.shape, ktf,
+                             ktf.shape, None, (False, False, False), np.float32, 1342177280, 2 * 5242880 + 33554432, 200, 1e-3))
     # C4's second half: the down-projection has 64 output tiles and K = 10240; with the workspace the
     # library asks for, its K is cut among four workgroups per tile (rt_matmul_enqueue_ws)
     rng = np.random.default_rng(6)

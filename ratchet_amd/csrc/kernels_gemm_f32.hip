@@ -9,8 +9,10 @@
 // tiles).  An f32 MFMA is slow (32 cycles for 2048 flop), so LDS and memory traffic are light and
 // the launcher picks the tile by how much the fixed costs weigh (see launch_gemm_f32).  K tile 32,
 // two LDS stages, one bare barrier per tile; tile t+1 waits in registers while tile t is multiplied
-// and tile t+2 is in flight.  K must be a whole number of tiles, which keeps the loop free of
-// branches (other K go to the generic kernel).
+// and tile t+2 is in flight.  With K a whole number of tiles the loop has no bound to check; other K
+// (a multiple of 4: attention scores over a head dimension of 80) run the KTAIL variant, whose loads
+// clamp their K offset and whose LDS stores write zeros past K -- selects, not branches, so the loop
+// stays straight-line code either way.
 //
 // LDS rows are padded so that every fragment read is conflict-free on 64 banks:
 //   [row][k] tiles, stride 36: lane (r = l % 16, q = l / 16) reads word 36 r + 4 kk + q; 36 r mod 64
@@ -40,7 +42,7 @@ constexpr int F32_LDA = F32_BK + 4;
 
 // B_KCONT: B's K axis is the contiguous one (its tile is [col][k], like A's); otherwise its
 // column axis is (tile [k][col]).
-template <int BM, int BN, bool B_KCONT>
+template <int BM, int BN, bool B_KCONT, bool KTAIL>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
     static_assert(WM % 16 == 0 && WN % 16 == 0, "a wavefront's share must split into 16 x 16 MFMA tiles");
@@ -71,24 +73,28 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     // their products land in outputs that are never stored).
     const float *pa[A_PT], *pb[B_PT];
     int la[A_PT], lb[B_PT]; // LDS word offsets
+    int ka[A_PT], kb[B_PT]; // K offset of the vector inside a tile (KTAIL)
 #pragma unroll
     for (int e = 0; e < A_PT; e++) {
         const int v = min(e * 256 + t, A_VECS - 1);
         const int row = v / (F32_BK / 4), c4 = v % (F32_BK / 4);
-        pa[e] = A + min(i0 + row, g.M - 1) * g.a_rs + 4 * c4;
+        pa[e] = A + min(i0 + row, g.M - 1) * g.a_rs + (KTAIL ? 0 : 4 * c4);
         la[e] = row * F32_LDA + 4 * c4;
+        ka[e] = 4 * c4;
     }
 #pragma unroll
     for (int e = 0; e < B_PT; e++) {
         const int v = min(e * 256 + t, B_VECS - 1);
         if constexpr (B_KCONT) {
             const int col = v / (F32_BK / 4), c4 = v % (F32_BK / 4);
-            pb[e] = B + min(j0 + col, g.N - 1) * g.b_js + 4 * c4;
+            pb[e] = B + min(j0 + col, g.N - 1) * g.b_js + (KTAIL ? 0 : 4 * c4);
             lb[e] = A_FLOATS + col * LDB + 4 * c4;
+            kb[e] = 4 * c4;
         } else {
             const int k = v / (BN / 4), c4 = v % (BN / 4);
-            pb[e] = B + (int64_t)k * g.b_ks + min(j0 + 4 * c4, g.N - 4); // N % 4 == 0: a vector is wholly in or out
+            pb[e] = B + (KTAIL ? 0 : (int64_t)k * g.b_ks) + min(j0 + 4 * c4, g.N - 4); // N % 4 == 0: a vector is wholly in or out
             lb[e] = A_FLOATS + k * LDB + 4 * c4;
+            kb[e] = k;
         }
     }
     struct Regs {
@@ -97,20 +103,27 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     // K is a whole number of tiles (the launcher checks): no load needs a bound, so the loop body is
     // straight-line code and the compiler's wait counts stay exact (a conditional load makes it wait
     // for every outstanding load at the next register it overwrites).
+    // KTAIL (K % 4 == 0, any number of tiles): a vector past K re-reads the last valid one (still no bound on
+    // the load) and is replaced by zeros on its way into LDS.
     auto load_tile = [&](int64_t k0, Regs &r) {
 #pragma unroll
-        for (int e = 0; e < A_PT; e++) r.a[e] = *(const float4_t *)(pa[e] + k0);
+        for (int e = 0; e < A_PT; e++) r.a[e] = *(const float4_t *)(pa[e] + (KTAIL ? min(k0 + ka[e], g.K - 4) : k0));
 #pragma unroll
-        for (int e = 0; e < B_PT; e++) r.b[e] = *(const float4_t *)(pb[e] + (B_KCONT ? k0 : k0 * g.b_ks));
+        for (int e = 0; e < B_PT; e++) {
+            if constexpr (!KTAIL) r.b[e] = *(const float4_t *)(pb[e] + (B_KCONT ? k0 : k0 * g.b_ks));
+            else if constexpr (B_KCONT) r.b[e] = *(const float4_t *)(pb[e] + min(k0 + kb[e], g.K - 4));
+            else r.b[e] = *(const float4_t *)(pb[e] + min(k0 + kb[e], g.K - 1) * g.b_ks);
+        }
     };
-    auto store_tile = [&](int stage, const Regs &r) {
+    auto store_tile = [&](int stage, int64_t k0, const Regs &r) {
         float *st = smem + stage * STAGE;
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int e = 0; e < A_PT; e++)
-            if (A_VECS % 256 == 0 || e * 256 + t < A_VECS) *(float4_t *)(st + la[e]) = r.a[e];
+            if (A_VECS % 256 == 0 || e * 256 + t < A_VECS) *(float4_t *)(st + la[e]) = (!KTAIL || k0 + ka[e] < g.K) ? r.a[e] : zero;
 #pragma unroll
         for (int e = 0; e < B_PT; e++)
-            if (B_VECS % 256 == 0 || e * 256 + t < B_VECS) *(float4_t *)(st + lb[e]) = r.b[e];
+            if (B_VECS % 256 == 0 || e * 256 + t < B_VECS) *(float4_t *)(st + lb[e]) = (!KTAIL || k0 + kb[e] < g.K) ? r.b[e] : zero;
     };
 
     float4_t acc[TM][TN];
@@ -123,11 +136,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     // the other stage after the MFMAs) and tile kt + 2 is on its way from memory: a load has two
     // tiles' worth of MFMAs (about 2 us) to arrive, a first-touch HBM latency.
     // Past the last tile the loads repeat it and the stores refill a stage nobody reads again: no branch.
-    const int64_t nk = g.K / F32_BK;
+    const int64_t nk = (g.K + F32_BK - 1) / F32_BK;
     Regs r0, r1;
     load_tile(0, r0);
     load_tile(min<int64_t>(1, nk - 1) * F32_BK, r1);
-    store_tile(0, r0);
+    store_tile(0, 0, r0);
     __syncthreads();
     auto k_tile = [&](int64_t kt, Regs &incoming, const Regs &waiting) {
         const int cur = (int)(kt & 1);
@@ -156,7 +169,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
                     acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[kk & 1][a], fb[kk & 1][b], acc[a][b], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        store_tile(cur ^ 1, waiting);
+        store_tile(cur ^ 1, min(kt + 1, nk - 1) * F32_BK, waiting);
         // The other stage is complete; this one may be overwritten in the next iteration.  A bare
         // barrier behind a wait for the LDS operations only: __syncthreads() would also wait for the
         // global loads that were just issued for tile kt + 2.
@@ -201,15 +214,20 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     });
 }
 
-template <int BM, int BN, bool B_KCONT>
-static hipError_t launch_f32(const GemmF32Args &g, int64_t stacks, hipStream_t st) {
+template <int BM, int BN, bool B_KCONT, bool KTAIL>
+static hipError_t launch_f32_kt(const GemmF32Args &g, int64_t stacks, hipStream_t st) {
     constexpr int LDB = B_KCONT ? F32_LDA : BN + 16;
     constexpr size_t lds = (size_t)2 * (BM * F32_LDA + (B_KCONT ? BN * F32_LDA : F32_BK * LDB)) * sizeof(float);
-    if (const hipError_t e = ensure_lds_limit<&gemm_f32_kernel<BM, BN, B_KCONT>>(); e != hipSuccess) return e;
+    if (const hipError_t e = ensure_lds_limit<&gemm_f32_kernel<BM, BN, B_KCONT, KTAIL>>(); e != hipSuccess) return e;
     const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     if (tiles > 0x7fffffff) return hipErrorNotSupported;
-    hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, B_KCONT>), dim3((unsigned)tiles, (unsigned)stacks), dim3(256), lds, st, g);
+    hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, B_KCONT, KTAIL>), dim3((unsigned)tiles, (unsigned)stacks), dim3(256), lds, st, g);
     return hipGetLastError();
+}
+
+template <int BM, int BN, bool B_KCONT>
+static hipError_t launch_f32(const GemmF32Args &g, int64_t stacks, hipStream_t st) {
+    return g.K % F32_BK == 0 ? launch_f32_kt<BM, BN, B_KCONT, false>(g, stacks, st) : launch_f32_kt<BM, BN, B_KCONT, true>(g, stacks, st);
 }
 
 RT_TUNABLE(g_gemm_f32_bm, 0);      // 32 or 96 forces that tile height (0 = by shape)
@@ -220,7 +238,7 @@ RT_TUNABLE(g_gemm_f32_disable, 0); // non-zero sends f32 problems to the generic
 hipError_t launch_gemm_f32(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
                            const DeviceInfo &dev) {
     if (g_gemm_f32_disable || p.a_dt != RT_F32 || p.act_dt != RT_F32) return hipErrorNotSupported;
-    if (p.a_ks != 1 || (p.b_ks != 1 && p.b_js != 1) || p.K < F32_BK || p.K % F32_BK != 0) return hipErrorNotSupported;
+    if (p.a_ks != 1 || (p.b_ks != 1 && p.b_js != 1) || p.K < 4 || p.K % 4 != 0) return hipErrorNotSupported;
     if (p.M < 48 || p.N < 48 || p.stacks > 65535) return hipErrorNotSupported; // small outputs: the generic 64 x 64 tiles
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)out) & 15u) return hipErrorNotSupported;
     if (p.a_rs % 4 || p.a_bs % 4 || p.b_bs % 4) return hipErrorNotSupported;

@@ -623,7 +623,10 @@ def test_f32_contiguous_operands(device, oracle):
     tile edges in both dimensions, K from one tile to many (both tile heights), stacks, broadcast, both bias axes."""
     #        S  M    N    K
     shapes = [(1, 48, 48, 32), (1, 97, 100, 64), (1, 1500, 1536, 384), (2, 130, 52, 96), (1, 50, 333, 1024),
-              (3, 200, 96, 800), (1, 96, 4000, 32)]
+              (3, 200, 96, 800), (1, 96, 4000, 32),
+              # K that is not a whole number of 32-wide tiles (any multiple of 4): the head dimension of 80 of the
+              # phi2 / whisper score product q.matmul(k.permute([0, 1, 3, 2]), false, false), shorter than a tile, ragged
+              (32, 512, 512, 80), (2, 100, 64, 4), (1, 60, 120, 20), (2, 129, 200, 100), (1, 96, 96, 36), (1, 300, 52, 1000)]
     for i, (S, M, N, K) in enumerate(shapes):
         rng = np.random.default_rng(1000 + i)
         a = (rng.standard_normal((S, M, K)) * 0.1).astype(np.float32)
