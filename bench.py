@@ -496,20 +496,7 @@ def other_configs(r: Runner, O):
     bias = (rng.standard_normal(1536) * 0.05).astype(np.float32)
     out.append(bench_generic(r, O, "C1 f32 GEMM [1500x384].[384x1536]+b", a, ffi.RT_F32, a.shape, b, b.shape, bias,
                              (False, False, False), np.float32, 1769472000, 13885440, 200, 1e-3))
-    rng = np.random.default_rng(1)
-    q = rng.standard_normal((1, 32, 512, 80)).astype(np.float16)
-    k = rng.standard_normal((1, 32, 512, 80)).astype(np.float16)
-    v = rng.standard_normal((1, 32, 512, 80)).astype(np.float16)
-    p = (rng.random((1, 32, 512, 512)) / 512).astype(np.float16)
-    out.append(bench_generic(r, O, "C3 QK^T f16 [32x512x80].[32x512x80]^T", q, ffi.RT_F16, q.shape, k, k.shape, None,
-                             (False, True, False), np.float16, 1342177280, 22020096, 200, 2e-2))
-    out.append(bench_generic(r, O, "C3 PV f16 [32x512x512].[32x512x80]", p, ffi.RT_F16, p.shape, v, v.shape, None,
-                             (False, False, False), np.float16, 1342177280, 22020096, 200, 2e-2))
-    # the phi2 / whisper spelling of the score product: f32 operands, the key permuted beforehand, matmul(false, false)
-    # (crates/ratchet-models/src/phi2/attn.rs:139-142): reads 2 x 5.2 MB, writes 33.6 MB of f32 scores
-    qf, ktf = q.astype(np.float32), np.ascontiguousarray(k.astype(np.float32).transpose(0, 1, 3, 2))
-    out.append(bench_generic(r, O, "C3 QK^T f32, key permuted beforehand [32x512x80].[32x80x512]", qf, ffi.RT_F32, qf.shape, ktf,
-                             ktf.shape, None, (False, False, False), np.float32, 1342177280, 2 * 5242880 + 33554432, 200, 1e-3))
+    out += c3_products(r, O)
     # C4's second half: the down-projection has 64 output tiles and K = 10240; with the workspace the
     # library asks for, its K is cut among four workgroups per tile (rt_matmul_enqueue_ws)
     rng = np.random.default_rng(6)
@@ -527,6 +514,26 @@ def other_configs(r: Runner, O):
     out.append(bench_decoder_layer(r, O))
     out.append(bench_decoder_layer(r, O, fused_qkv=True))
     out += bench_q4k(r, O, (1, 16, 256), 200)
+    return out
+
+
+def c3_products(r: Runner, O):
+    """BASELINE configs[2]: the two attention products at 32 heads x 512 x 80, f16, and the f32 spelling of the first."""
+    ffi, out = r.ffi, []
+    rng = np.random.default_rng(1)
+    q = rng.standard_normal((1, 32, 512, 80)).astype(np.float16)
+    k = rng.standard_normal((1, 32, 512, 80)).astype(np.float16)
+    v = rng.standard_normal((1, 32, 512, 80)).astype(np.float16)
+    p = (rng.random((1, 32, 512, 512)) / 512).astype(np.float16)
+    out.append(bench_generic(r, O, "C3 QK^T f16 [32x512x80].[32x512x80]^T", q, ffi.RT_F16, q.shape, k, k.shape, None,
+                             (False, True, False), np.float16, 1342177280, 22020096, 200, 2e-2))
+    out.append(bench_generic(r, O, "C3 PV f16 [32x512x512].[32x512x80]", p, ffi.RT_F16, p.shape, v, v.shape, None,
+                             (False, False, False), np.float16, 1342177280, 22020096, 200, 2e-2))
+    # the phi2 / whisper spelling of the score product: f32 operands, the key permuted beforehand, matmul(false, false)
+    # (crates/ratchet-models/src/phi2/attn.rs:139-142): reads 2 x 5.2 MB, writes 33.6 MB of f32 scores
+    qf, ktf = q.astype(np.float32), np.ascontiguousarray(k.astype(np.float32).transpose(0, 1, 3, 2))
+    out.append(bench_generic(r, O, "C3 QK^T f32, key permuted beforehand [32x512x80].[32x80x512]", qf, ffi.RT_F32, qf.shape, ktf,
+                             ktf.shape, None, (False, False, False), np.float32, 1342177280, 2 * 5242880 + 33554432, 200, 1e-3))
     return out
 
 
@@ -615,6 +622,8 @@ def main():
     ap.add_argument("--no-secondary", action="store_true", help="only the headline workload")
     ap.add_argument("--gemm-only", action="store_true",
                     help="run only the two C4 GEMM workloads (f16 and Q8_0H weights) and print their lines; for profiling")
+    ap.add_argument("--c3-only", action="store_true",
+                    help="run only the attention products of configs[2] and print their lines; for profiling")
     ap.add_argument("--q4k-only", action="store_true",
                     help="run only the Q4_K prefill workload (C5 at 256 rows) and print its line; for profiling")
     ap.add_argument("--read-calibration", action="store_true",
@@ -650,6 +659,11 @@ def main():
                   bench_f16_gemm(r, O, 50, 5, M=4096)):
             print(json.dumps({"workload": g["workload"], "tflops": round(g["tflops"], 1), "ms_per_step": g["ms"],
                               "frac_mfma_f16_peak": round(g["tflops"] / MFMA_F16_PEAK_TFLOPS, 4)}))
+        return 0
+
+    if args.c3_only:
+        for g in c3_products(r, O):
+            print(json.dumps(g))
         return 0
 
     if args.q4k_only:

@@ -2,15 +2,25 @@
 // (+ bias), A rows K-contiguous, B rows N-contiguous, N <= 128, C row-major.  This is the
 // attention P.V form (P [seq x seq], V [seq x head_dim]): a stream over A, read exactly once.
 //
-// A workgroup of four wavefronts owns 32 rows of A and all of N.  Per K tile of 64 the A tile
-// goes global -> registers -> LDS as it is.  The B tile (64 x N) is copied row by row with
-// fully coalesced 16-byte loads (fetching 8 x 8 blocks straight from global memory, 16 bytes
-// per row, measured 7 us slower on the attention shape) and transposed inside LDS: a thread
-// reads an 8 x 8 block as eight 16-byte rows, exchanges halves with 32 v_perm_b32 and writes
-// eight 16-byte columns, so LDS holds B as [n][k] and both MFMA operands are single 128-bit
-// fragment reads.  The loads of the next three tiles are in flight under the MFMAs.  A wavefront
-// multiplies 16 rows by half of the 16-column tiles of B (v_mfma_f32_16x16x32_f16), stages its
-// result in LDS and writes it with 128-bit stores.
+// A workgroup of eight wavefronts owns 64 rows of A and all of N.  A is used once, so it never
+// touches LDS: lane (fr, fg) loads the 16 bytes A[row fr][32 kh + 8 fg ..] that are its operand
+// of a K step.  B is shared by the workgroup and goes through LDS as it lies in memory, [k][n]:
+// ds_read_b64_tr_b16 hands each lane the four consecutive k of one column that an MFMA operand
+// wants (within 16 lanes, lane s addresses columns 4 (s % 4) .. + 3 of row s / 4 and lane i
+// receives column i of the four rows), so nothing is transposed by hand.  Per K tile of 64 the
+// wavefronts 0..3 multiply their 16 rows by the tile's first 32 rows of B and the wavefronts 4..7
+// by the other 32 (v_mfma_f32_16x16x32_f16); the two partial sums meet in LDS at the end.  Two LDS
+// stages, one barrier per tile; the loads of the next seven tiles are in flight in registers: at
+// the sizes this kernel sees (a few tens of MB) the whole problem has to be requested at once to
+// keep HBM busy.  The result is staged in LDS and written with 128-bit stores.
+//
+// EXACT: M and K are multiples of 64, N of 16 and a workgroup's operands span less than 2 GiB: no
+// clamps or zero fills, and every load is a wave-uniform base plus a 32-bit lane offset fixed for
+// the whole kernel.
+//
+// Measured on the attention shape (32 x [512 x 512] . [512 x 80], 22 MB): loads alone 8.5 us, of
+// which A alone 7.6 (6.8 if a wavefront read whole rows instead of 16 rows x 64 bytes), LDS stores
+// and barriers + 0.3, transposing reads and MFMAs + 1.4; the arithmetic alone, without the loads, 4.1.
 //
 // Role in the reference: ops/gemm.rs:305-657 with trans_rhs = false (phi2 / whisper attention,
 // `matmul(V, false, false)`).
@@ -29,156 +39,179 @@ struct GemmNnArgs {
     int has_bias, bias_on_rows, act;
 };
 
-constexpr int NN_THREADS = 256, NN_BM = 32, NN_BK = 64, NN_DEPTH = 4;
-constexpr int NN_LDK = NN_BK + 8; // halfs per LDS row: 9 slots of 16 bytes, conflict-free fragment reads
+constexpr int NN_BK = 64;
 
-// TN: 16-column tiles of B (N <= 16 * TN).  Four wavefronts: two groups of 16 A rows times two
-// halves of the column tiles.
-template <int TN>
-__global__ __launch_bounds__(NN_THREADS) void gemm_nn_smalln_kernel(GemmNnArgs g) {
+constexpr int NNT_BM = 64, NNT_DEPTH = 8, NNT_THREADS = 512;
+
+template <int TN, bool EXACT>
+__global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr_kernel(GemmNnArgs g) {
     constexpr int NP = 16 * TN;                        // padded N
-    constexpr int TH = (TN + 1) / 2;                   // column tiles of the first half (the second has TN - TH)
-    constexpr int NBLK = (NN_BK / 8) * (NP / 8);       // 8 x 8 blocks of the B tile
-    static_assert(NBLK <= NN_THREADS && NN_BM * (NN_BK / 8) == NN_THREADS, "one A vector and at most one B block per thread");
-    constexpr int EROW = 16 * TH + 8;
-    constexpr int BR = NP + 8;                         // halfs per row of the untransposed B tile (odd number of 16-byte slots)
-    constexpr int B_VEC = (NN_BK * (NP / 8) + NN_THREADS - 1) / NN_THREADS; // 16-byte vectors of the B tile per thread
+    constexpr int BR = NP + 8;                         // halfs per row of the B tile
+    constexpr int B_VECS = NN_BK * (NP / 8);           // 16-byte vectors of a full B tile
+    constexpr int B_VEC = (B_VECS + NNT_THREADS - 1) / NNT_THREADS; // per thread
+    constexpr int STAGE = NN_BK * BR;
+    constexpr int EROW = NP + 8;
+    constexpr int RED_FLOATS = 4 * TN * 4 * 64;        // the second wavefront group's accumulators
+    static_assert(NN_BK == 64, "two K steps per tile, one per wavefront group");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    half_t *As = (half_t *)smem;        // [32][NN_LDK]
-    half_t *Bt = As + NN_BM * NN_LDK;   // [NP][NN_LDK]: B transposed
-    half_t *Br = Bt + NP * NN_LDK;      // [64][BR]: the B tile as it lies in memory
-    half_t *Es = Br;                    // [4 wavefronts][16][EROW]: output staging, after the K loop
-    static_assert(4 * 16 * EROW <= NN_BK * BR, "output staging reuses the untransposed B tile");
+    half_t *S0 = (half_t *)smem; // [2][64][BR]; afterwards the partial sums [4][TN][4][64] f32 and the output staging
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int rg = wave >> 1, nh = wave & 1;            // row group, column half
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int rw = wave & 3, kh = wave >> 2; // 16 rows of A, and which K step of every tile
     const int fr = lane & 15, fg = lane >> 4;
-    const int64_t i0 = (int64_t)blockIdx.x * NN_BM;
-    const int64_t s = blockIdx.y;
+    // Workgroups go to the eight XCDs round robin by their linear index, and each XCD has its own L2:
+    // the row blocks of one stack share its B, so they are given indices that land on one XCD.
+    const uint32_t mb = (uint32_t)((g.M + NNT_BM - 1) / NNT_BM), nstacks = gridDim.x / mb;
+    uint32_t blk = blockIdx.x % mb, stk = blockIdx.x / mb;
+    if (nstacks % 8 == 0) {
+        const uint32_t idx = blockIdx.x >> 3;
+        stk = (blockIdx.x & 7) + 8 * (idx / mb), blk = idx % mb;
+    }
+    const int64_t i0 = (int64_t)blk * NNT_BM;
+    const int64_t s = stk;
     const half_t *A = g.A + (g.a_stack == 1 ? 0 : s) * g.a_bs;
     const half_t *B = g.B + (g.b_stack == 1 ? 0 : s) * g.b_bs;
-    const int nvec = (int)(g.N >> 3); // 16-byte vectors per B row
+    const int nvec = EXACT ? NP / 8 : (int)(g.N >> 3);
     const uint4_t zero4 = {0u, 0u, 0u, 0u};
 
-    // this thread's A vector (row ar, K vector ac) and B block (K rows 8 kb.., columns 8 nb..)
-    const int ar = t >> 3, ac = t & 7;
-    const int blk = min(t, NBLK - 1), kb = blk & 7, nb = blk >> 3;
-    const bool b_live = t < NBLK && nb < nvec; // blocks past N are never written: those columns are never stored
-    const half_t *ap = A + min(i0 + ar, g.M - 1) * g.a_rs + 8 * ac; // rows past the end duplicate the last one
-    // this thread's vectors of the untransposed B tile: vector v = t + 256 i is (row v / nvec, column 8 (v % nvec))
+    // this lane's row of A (rows past the end duplicate the last one), its K offset inside a tile, and
+    // its vectors of the B tile: vector v = t + 512 i is (row v / nvec, column 8 (v % nvec))
+    const int arow = rw * 16 + fr, ak = 32 * kh + 8 * fg;
+    const half_t *ap = A + min(i0 + arow, g.M - 1) * g.a_rs + ak;
     int bk[B_VEC], bc[B_VEC];
 #pragma unroll
     for (int i = 0; i < B_VEC; i++) {
-        const int v = min(t + NN_THREADS * i, NN_BK * nvec - 1);
+        const int v = min(t + NNT_THREADS * i, NN_BK * nvec - 1);
         bk[i] = v / nvec, bc[i] = v - bk[i] * nvec;
     }
+    // EXACT: byte offsets from the tile's first byte
+    const uint32_t aoff = 2u * (uint32_t)(arow * (int)g.a_rs + ak);
+    uint32_t boff[B_VEC];
+#pragma unroll
+    for (int i = 0; i < B_VEC; i++) boff[i] = 2u * (uint32_t)(bk[i] * (int)g.b_ks + 8 * bc[i]);
+    const char *abase = (const char *)(A + i0 * g.a_rs);
+    const int64_t b_tile_bytes = 2 * NN_BK * g.b_ks;
+    auto b_mine = [&](int i) { return NNT_THREADS * (i + 1) <= B_VECS || t + NNT_THREADS * i < (EXACT ? B_VECS : NN_BK * nvec); };
 
-    // D register sets: the loads of the next D - 1 tiles are in flight while one is multiplied
-    // (a tile's MFMAs are far shorter than a trip to HBM)
-    constexpr int D = NN_DEPTH;
+    constexpr int D = NNT_DEPTH;
     uint4_t ra_[D], rb_[D][B_VEC];
     auto load_tiles = [&](int64_t k0, uint4_t &ra, uint4_t (&rb)[B_VEC]) {
-        ra = *(const uint4_t *)(ap + min(k0, g.K - 8 - 8 * ac)); // vectors past K re-read a valid one; zeroed below
+        if constexpr (EXACT) {
+            const char *at = abase + 2 * k0, *bt = (const char *)B + (k0 / NN_BK) * b_tile_bytes; // uniform
 #pragma unroll
-        for (int i = 0; i < B_VEC; i++) rb[i] = *(const uint4_t *)(B + min(k0 + bk[i], g.K - 1) * g.b_ks + 8 * bc[i]);
+            for (int i = 0; i < B_VEC; i++) rb[i] = *(const uint4_t *)(bt + boff[i]); // (threads without a vector re-read the last one)
+            ra = *(const uint4_t *)(at + aoff);
+        } else {
+#pragma unroll
+            for (int i = 0; i < B_VEC; i++) rb[i] = *(const uint4_t *)(B + min(k0 + bk[i], g.K - 1) * g.b_ks + 8 * bc[i]);
+            const uint4_t v = *(const uint4_t *)(ap + min(k0, g.K - 8 - ak)); // past K: a valid vector, replaced by zeros
+            ra = k0 + ak < g.K ? v : zero4;
+        }
     };
-    // registers -> LDS: A as it is, B rows as they are (rows past K zeroed, so the padded part of
-    // the last K tile adds nothing)
-    auto store_tiles = [&](int64_t k0, const uint4_t &ra, const uint4_t (&rb)[B_VEC]) {
-        const bool full = k0 + NN_BK <= g.K; // uniform: only the last tile can be ragged
-        *(uint4_t *)(As + ar * NN_LDK + 8 * ac) = (full || k0 + 8 * ac < g.K) ? ra : zero4;
+    // registers -> LDS: B rows as they are (rows past K zeroed: the padded part of the last K tile adds nothing)
+    auto store_tile = [&](half_t *st, int64_t k0, const uint4_t (&rb)[B_VEC]) {
+        const bool full = EXACT || k0 + NN_BK <= g.K; // uniform: only the last tile can be ragged
 #pragma unroll
         for (int i = 0; i < B_VEC; i++)
-            if (t + NN_THREADS * i < NN_BK * nvec)
-                *(uint4_t *)(Br + bk[i] * BR + 8 * bc[i]) = (full || k0 + bk[i] < g.K) ? rb[i] : zero4;
-    };
-    // Br [k][n] -> Bt [n][k]: column c of an 8 x 8 block = halves c of its rows 0..7
-    auto transpose_b = [&]() {
-        if (b_live) {
-            uint4_t row[8];
-#pragma unroll
-            for (int r = 0; r < 8; r++) row[r] = *(const uint4_t *)(Br + (8 * kb + r) * BR + 8 * nb);
-#pragma unroll
-            for (int c = 0; c < 8; c++) {
-                uint4_t col;
-#pragma unroll
-                for (int m = 0; m < 4; m++)
-                    col[m] = __builtin_amdgcn_perm(row[2 * m + 1][c >> 1], row[2 * m][c >> 1],
-                                                   (c & 1) ? 0x07060302u : 0x05040100u);
-                *(uint4_t *)(Bt + (8 * nb + c) * NN_LDK + 8 * kb) = col;
-            }
-        }
+            if (b_mine(i)) *(uint4_t *)(st + bk[i] * BR + 8 * bc[i]) = (full || k0 + bk[i] < g.K) ? rb[i] : zero4;
     };
 
-    float4_t acc[TH];
+    float4_t acc[TN];
 #pragma unroll
-    for (int b = 0; b < TH; b++) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
-    const int b0 = nh * TH, nb_tiles = nh == 0 ? TH : TN - TH; // this wavefront's column tiles
-    const int64_t nk = (g.K + NN_BK - 1) / NN_BK;
+    for (int b = 0; b < TN; b++) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+    // byte address in LDS of the first row / columns this lane addresses for B
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const half_t *)S0;
+    const uint32_t b_off = lds0 + 2u * (uint32_t)((32 * kh + 8 * fg + (fr >> 2)) * BR + 4 * (fr & 3));
+
+    const int nk = (int)((g.K + NN_BK - 1) / NN_BK);
+    auto tile_k0 = [&](int kt) { return (int64_t)kt * NN_BK; };
+    // (unconditional: a branch here would leave the compiler unable to count the loads in flight, and it
+    // would then wait for all of them before the first tile; short problems load their last tile again)
 #pragma unroll
-    for (int d = 0; d < D - 1; d++)
-        if (d < nk) load_tiles((int64_t)d * NN_BK, ra_[d], rb_[d]);
-    for (int64_t kt0 = 0; kt0 < nk; kt0 += D) {
+    for (int d = 0; d < D - 1; d++) {
+        load_tiles(tile_k0(min(d, nk - 1)), ra_[d], rb_[d]);
+        __builtin_amdgcn_sched_barrier(0); // in this order: the first tile's data is waited for first
+    }
+    auto trip = [&](int kt0) {
 #pragma unroll
         for (int u = 0; u < D; u++) {
-            const int64_t kt = kt0 + u;
+            const int kt = kt0 + u;
             if (kt < nk) { // uniform
-                if (kt + D - 1 < nk) load_tiles((kt + D - 1) * NN_BK, ra_[(u + D - 1) % D], rb_[(u + D - 1) % D]);
-                store_tiles(kt * NN_BK, ra_[u], rb_[u]);
+                if (kt + D - 1 < nk) load_tiles(tile_k0(kt + D - 1), ra_[(u + D - 1) % D], rb_[(u + D - 1) % D]);
+                store_tile(S0 + (u & 1) * STAGE, tile_k0(kt), rb_[u]); // D is even: tile kt lives in stage kt % 2
+                // everybody's stores of this tile are done; everybody has finished with the other stage's last tile
                 __syncthreads();
-                transpose_b();
-                __syncthreads();
+                const uint32_t sb = b_off + 2u * (uint32_t)((u & 1) * STAGE);
+                uint64_t lo[TN], hi[TN];
 #pragma unroll
-                for (int kk = 0; kk < NN_BK / 32; kk++) {
-                    const half8_t fa = __builtin_bit_cast(half8_t, *(const uint4_t *)(As + (rg * 16 + fr) * NN_LDK + kk * 32 + 8 * fg));
-                    half8_t fb[TH];
+                for (int b = 0; b < TN; b++)
+                    asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                                 : "=&v"(lo[b]), "=&v"(hi[b])
+                                 : "v"(sb), "n"(2 * 16 * b), "n"(2 * (16 * b + 4 * BR))
+                                 : "memory");
 #pragma unroll
-                    for (int b = 0; b < TH; b++)
-                        fb[b] = __builtin_bit_cast(half8_t, *(const uint4_t *)(Bt + (min(b0 + b, TN - 1) * 16 + fr) * NN_LDK + kk * 32 + 8 * fg));
-                    // first operand: A rows (result registers), second: B columns (result lanes)
+                for (int b = 0; b < TN; b++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[b]), "+v"(hi[b])::"memory");
+                typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
+                const half8_t fa = __builtin_bit_cast(half8_t, ra_[u]);
 #pragma unroll
-                    for (int b = 0; b < TH; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, fb[b], acc[b], 0, 0, 0);
-                }
-                __syncthreads();
+                for (int b = 0; b < TN; b++)
+                    acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, __builtin_bit_cast(half8_t, u64x2_t{lo[b], hi[b]}), acc[b], 0, 0, 0);
             }
         }
-    }
+    };
+    // The first D tiles stand outside the loop: at a loop header the compiler's count of loads in flight
+    // is the cautious merge of both ways in, and it would wait for all of them before the first tile.
+    trip(0);
+    for (int kt0 = D; kt0 < nk; kt0 += D) trip(kt0);
+    __syncthreads(); // the stages become the partial sums and the output staging
 
-    // acc[b][r] is row 4 * fg + r of the wavefront's 16, column 16 * (b0 + b) + fr
-    half_t *es = Es + wave * 16 * EROW;
+    // the second group hands its sums to the first
+    float4_t *red = (float4_t *)smem + rw * TN * 64;
+    if (kh == 1) {
+#pragma unroll
+        for (int b = 0; b < TN; b++) red[b * 64 + lane] = acc[b];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+#pragma unroll
+    for (int b = 0; b < TN; b++) acc[b] += red[b * 64 + lane];
+
+    // acc[b][r] is row 4 * fg + r of the wavefront's 16, column 16 * b + fr
+    half_t *es = (half_t *)(smem + 4 * RED_FLOATS) + rw * 16 * EROW;
     rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
-        for (int b = 0; b < TH; b++) {
-            const int n = 16 * (b0 + b) + fr;
+        for (int b = 0; b < TN; b++) {
+            const int n = 16 * b + fr;
             float bn = 0.f;
             if (g.has_bias && !g.bias_on_rows) bn = (float)g.bias[min(n, (int)g.N - 1)];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int il = 4 * fg + r;
                 float v = acc[b][r] + bn;
-                if (g.has_bias && g.bias_on_rows) v += (float)g.bias[min(i0 + rg * 16 + il, g.M - 1)];
+                if (g.has_bias && g.bias_on_rows) v += (float)g.bias[min(i0 + rw * 16 + il, g.M - 1)];
                 v = rt_act_k<decltype(has_act)::value>(v);
-                es[il * EROW + 16 * b + fr] = (half_t)v;
+                es[il * EROW + n] = (half_t)v;
             }
         }
     });
     asm volatile("" ::: "memory"); // read back by the same wavefront; DS operations complete in order
     half_t *out = g.out + s * g.o_bs;
-    const int wvec = 2 * nb_tiles; // 16-byte vectors per row in this wavefront's columns
-    for (int v = lane; v < 16 * wvec; v += 64) {
-        const int il = v / wvec, c = v - il * wvec;
-        const int64_t i = i0 + rg * 16 + il;
-        const int n = 16 * b0 + 8 * c;
-        if (i < g.M && n < g.N) *(uint4_t *)(out + i * g.o_is + n) = *(const uint4_t *)(es + il * EROW + 8 * c);
+    for (int v = lane; v < 16 * nvec; v += 64) {
+        const int il = v / nvec, c = v - il * nvec;
+        const int64_t i = i0 + rw * 16 + il;
+        if (i < g.M) *(uint4_t *)(out + i * g.o_is + 8 * c) = *(const uint4_t *)(es + il * EROW + 8 * c);
     }
 }
 
-template <int TN> static hipError_t launch_nn_one(const GemmNnArgs &g, int64_t stacks, hipStream_t st) {
+template <int TN> static hipError_t launch_nn_tr(const GemmNnArgs &g, int64_t stacks, hipStream_t st) {
     constexpr int NP = 16 * TN;
-    const size_t lds = ((size_t)(NN_BM + NP) * NN_LDK + (size_t)NN_BK * (NP + 8)) * 2;
-    dim3 grid((unsigned)((g.M + NN_BM - 1) / NN_BM), (unsigned)stacks);
-    hipLaunchKernelGGL((gemm_nn_smalln_kernel<TN>), grid, dim3(NN_THREADS), lds, st, g);
+    const size_t lds = std::max<size_t>((size_t)2 * NN_BK * (NP + 8) * 2, (size_t)4 * 4 * TN * 4 * 64 + (size_t)4 * 16 * (NP + 8) * 2);
+    dim3 grid((unsigned)((g.M + NNT_BM - 1) / NNT_BM * stacks));
+    const bool exact = g.M % NNT_BM == 0 && g.K % NN_BK == 0 && g.N == NP && g.a_rs < (1 << 23) && g.K * g.b_ks < (1 << 29);
+    if (exact) hipLaunchKernelGGL((gemm_nn_tr_kernel<TN, true>), grid, dim3(NNT_THREADS), lds, st, g);
+    else hipLaunchKernelGGL((gemm_nn_tr_kernel<TN, false>), grid, dim3(NNT_THREADS), lds, st, g);
     return hipGetLastError();
 }
 
@@ -192,7 +225,7 @@ hipError_t launch_gemm_nn_smalln(const Problem &p, const void *A, const void *B,
     if (p.a_dt != RT_F16 || p.act_dt != RT_F16) return hipErrorNotSupported;
     if (p.a_ks != 1 || p.b_js != 1 || p.o_js != 1) return hipErrorNotSupported;
     if (p.N < 8 || p.N > 128 || p.N % 8 != 0 || p.K < 8 || p.K % 8 != 0 || p.M < 64) return hipErrorNotSupported;
-    if (p.stacks > 65535 || (p.M + NN_BM - 1) / NN_BM > 0x7fffffff) return hipErrorNotSupported;
+    if (p.stacks > 65535 || (p.M + NNT_BM - 1) / NNT_BM * p.stacks > 0x7fffffff) return hipErrorNotSupported;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || ((uintptr_t)out & 15u)) return hipErrorNotSupported;
     if (p.a_rs % 8 || p.a_bs % 8 || p.b_ks % 8 || p.b_bs % 8 || p.o_is % 8 || p.o_bs % 8) return hipErrorNotSupported;
     GemmNnArgs g{};
@@ -205,14 +238,14 @@ hipError_t launch_gemm_nn_smalln(const Problem &p, const void *A, const void *B,
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
     const int tn = (int)((p.N + 15) / 16);
     switch (tn) {
-    case 1: return launch_nn_one<1>(g, p.stacks, stream);
-    case 2: return launch_nn_one<2>(g, p.stacks, stream);
-    case 3: return launch_nn_one<3>(g, p.stacks, stream);
-    case 4: return launch_nn_one<4>(g, p.stacks, stream);
-    case 5: return launch_nn_one<5>(g, p.stacks, stream);
-    case 6: return launch_nn_one<6>(g, p.stacks, stream);
-    case 7: return launch_nn_one<7>(g, p.stacks, stream);
-    default: return launch_nn_one<8>(g, p.stacks, stream);
+    case 1: return launch_nn_tr<1>(g, p.stacks, stream);
+    case 2: return launch_nn_tr<2>(g, p.stacks, stream);
+    case 3: return launch_nn_tr<3>(g, p.stacks, stream);
+    case 4: return launch_nn_tr<4>(g, p.stacks, stream);
+    case 5: return launch_nn_tr<5>(g, p.stacks, stream);
+    case 6: return launch_nn_tr<6>(g, p.stacks, stream);
+    case 7: return launch_nn_tr<7>(g, p.stacks, stream);
+    default: return launch_nn_tr<8>(g, p.stacks, stream);
     }
 }
 
