@@ -41,6 +41,10 @@ INFINITY_CACHE_BYTES = 256 << 20
 # readings are in profiles/gemv_q8_phi2_m1_pmc.txt.  A counter reading cannot be taken inside
 # this script, so the figure is the recorded one for the M=1 workload.
 GEMV_TRAFFIC_BYTES = 28149248
+# The same for the f16 GEMM of the metric's second half (profiles/gemm_c4_f16_q8_pmc.txt): FETCH_SIZE
+# 36,020 KiB x 1.99982 (copy calibration) + WRITE_SIZE 10,240 KiB.  The weight is read once and the
+# activations once per XCD (eight L2s), which is what puts it above the 65.6 MB the shape holds.
+GEMM_F16_TRAFFIC_BYTES = 84248078
 
 
 def gemv_bytes(M, N, K):
@@ -674,6 +678,9 @@ def main():
     wbuf, x, bias = head.pop("inputs")
     (cpu_s, cpu_n), (cpu_am_s, cpu_am_n) = cpu_baseline(O, wbuf, x, bias)
 
+    # the metric's second half (f16 GEMM at the configs[3] shape) always runs: its roofline object is part of the line
+    gemm_f16 = bench_f16_gemm(r, O, max(50, args.steps // 40), 10)
+
     secondary = []
     if not args.no_secondary:
         sec_steps = max(200, args.steps // 4)
@@ -687,7 +694,7 @@ def main():
             secondary.append({"workload": f"C2 Q8_0 GEMV M={M}", "value": round(s["gbps"], 1), "unit": "GB/s",
                               "ms_per_step": s["ms"], "frac_hbm_peak": round(s["gbps"] / HBM_PEAK_GBPS, 4)})
         gsteps = max(50, args.steps // 40)
-        for g in (bench_f16_gemm(r, O, gsteps, 10), bench_q8_gemm(r, O, gsteps, 10),
+        for g in (gemm_f16, bench_q8_gemm(r, O, gsteps, 10),
                   bench_q8_gemm(r, O, gsteps, 10, act=r.ffi.RT_ACT_GELU)):
             secondary.append({"workload": g["workload"], "value": round(g["tflops"], 1), "unit": "TFLOP/s",
                               "ms_per_step": g["ms"], "frac_mfma_f16_peak": round(g["tflops"] / MFMA_F16_PEAK_TFLOPS, 4)})
@@ -728,6 +735,19 @@ def main():
             "traffic": GEMV_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": head["bytes"],
             "kernel": "gemv_q8h_rowdot_kernel<5, 1, 1>",
+        },
+        "roofline_gemm": {
+            "workload": gemm_f16["workload"],
+            "bound": "mfma",
+            "achieved": round(gemm_f16["tflops"], 1),
+            "peak": MFMA_F16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(gemm_f16["tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+            "traffic": GEMM_F16_TRAFFIC_BYTES,
+            "algorithmic_flops_per_launch": gemm_f16["flops"],
+            "algorithmic_bytes_per_launch": gemm_f16["bytes"],
+            "ms_per_step": gemm_f16["ms"],
+            "kernel": "gemm_nt_dl_kernel<160, 128, 3, 2>",
         },
         "cpu_baseline": {
             "value": round(head["bytes"] / cpu_s / 1e9, 3),
