@@ -5,8 +5,8 @@
 // weights).  v_mfma_f32_16x16x4_f32 takes one f32 per lane and operand, so neither tile needs a
 // transpose: A sits in LDS as [row][k] and B as it lies in memory, [k][col] or [col][k].
 //
-// 96 x 96 or 32 x 96 outputs per 256-thread workgroup (2 x 2 wavefronts of 3 x 3 or 1 x 3 MFMA
-// tiles).  An f32 MFMA is slow (32 cycles for 2048 flop), so LDS and memory traffic are light and
+// 128 x 128, 96 x 96 or 32 x 96 outputs per 256-thread workgroup (2 x 2 wavefronts of 4 x 4, 3 x 3 or
+// 1 x 3 MFMA tiles).  An f32 MFMA is slow (32 cycles for 2048 flop), so LDS and memory traffic are light and
 // the launcher picks the tile by how much the fixed costs weigh (see launch_gemm_f32).  K tile 32,
 // two LDS stages, one bare barrier per tile; tile t+1 waits in registers while tile t is multiplied
 // and tile t+2 is in flight.  With K a whole number of tiles the loop has no bound to check; other K
@@ -157,16 +157,19 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
 #pragma unroll
             for (int b = 0; b < TN; b++) fb[set][b] = B_KCONT ? bs[b * 16 * LDB + 4 * kk] : bs[4 * kk * LDB + b * 16];
         };
+        const int klen = KTAIL ? (int)min<int64_t>(F32_BK, g.K - kt * F32_BK) : F32_BK; // the last tile may be short
         read_step(0, 0);
 #pragma unroll
         for (int kk = 0; kk < F32_BK / 4; kk++) {
             if (kk + 1 < F32_BK / 4) read_step(kk + 1, (kk + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
+            if (!KTAIL || 4 * kk < klen) { // uniform: the zeros past K are not multiplied
 #pragma unroll
-            for (int a = 0; a < TM; a++)
+                for (int a = 0; a < TM; a++)
 #pragma unroll
-                for (int b = 0; b < TN; b++)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[kk & 1][a], fb[kk & 1][b], acc[a][b], 0, 0, 0);
+                    for (int b = 0; b < TN; b++)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[kk & 1][a], fb[kk & 1][b], acc[a][b], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         store_tile(cur ^ 1, min(kt + 1, nk - 1) * F32_BK, waiting);
@@ -258,7 +261,13 @@ hipError_t launch_gemm_f32(const Problem &p, const void *A, const void *B, const
     // K = 384); 96-row tiles read less LDS per MFMA and win from K of about 1000 on (78 against 81 us at 1536).
     const int64_t tiles96 = ((p.M + 95) / 96) * ((p.N + 95) / 96) * p.stacks;
     int bm = (p.K <= 768 || tiles96 < dev.num_cus) ? 32 : 96;
-    if (g_gemm_f32_bm == 32 || g_gemm_f32_bm == 96) bm = g_gemm_f32_bm;
+    // Short contractions (attention scores spelled [.., M, K] . [.., K, N], K = 80): nearly all the time goes
+    // into fetching operands and writing the output, so the largest tile wins while it still gives every
+    // compute unit two workgroups (25.4 against 30.6 us at 32 x [512 x 80] . [80 x 512]).
+    const int64_t tiles128 = ((p.M + 127) / 128) * ((p.N + 127) / 128) * p.stacks;
+    if (p.K <= 128 && tiles128 >= 2 * (int64_t)dev.num_cus) bm = 128;
+    if (g_gemm_f32_bm == 32 || g_gemm_f32_bm == 96 || g_gemm_f32_bm == 128) bm = g_gemm_f32_bm;
+    if (bm == 128) return b_kcont ? launch_f32<128, 128, true>(g, p.stacks, stream) : launch_f32<128, 128, false>(g, p.stacks, stream);
     if (bm == 32) return b_kcont ? launch_f32<32, 96, true>(g, p.stacks, stream) : launch_f32<32, 96, false>(g, p.stacks, stream);
     return b_kcont ? launch_f32<96, 96, true>(g, p.stacks, stream) : launch_f32<96, 96, false>(g, p.stacks, stream);
 }
