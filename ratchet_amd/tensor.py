@@ -320,6 +320,11 @@ FUSE_ACTIVATIONS = True
 # it asks for; False keeps every product in one pass.
 SPLIT_K = True
 
+# Checked mode (the role of the reference's RATCHET_CHECKED, gpu/pools/kernel_module_pool.rs:62-67): every
+# output buffer is filled with 0xFF bytes (NaN as f16 and as f32) before the operator that writes it is
+# enqueued, so an element a kernel fails to write cannot pass for a number.  The GPU tests switch it on.
+POISON_OUTPUTS = False
+
 
 class Tensor:
     """Lazy tensor: either resolved storage, or an operator node awaiting resolve()."""
@@ -497,6 +502,8 @@ class Tensor:
             return
         esz = 4 if self.dt == DType.F32 else 2
         out = torch.empty(max(self.numel() * esz, 16), dtype=torch.uint8, device=f"cuda:{dev.ordinal}")
+        if POISON_OUTPUTS:
+            out.fill_(0xFF)
         if isinstance(op, Cache):
             B, H, cap, D = op.cache.shape
             strides = (ctypes.c_int64 * 3)(*op.src_strides)

@@ -21,8 +21,11 @@ def oracle():
 
 @pytest.fixture(scope="session")
 def device():
-    """Device::request_device(DeviceRequest::GPU); GPU tests fail loudly without it."""
+    """Device::request_device(DeviceRequest::GPU); GPU tests fail loudly without it.  Every GPU test runs in
+    checked mode: outputs are NaN-filled before the operator that writes them is enqueued."""
+    import ratchet_amd.tensor as mirror
     from ratchet_amd import Device, DeviceRequest
+    mirror.POISON_OUTPUTS = True
     return Device.request_device(DeviceRequest.GPU)
 
 

@@ -745,3 +745,28 @@ def test_quantized_weights_a_few_more_vectors_than_one_streaming_launch(device, 
             got = gpu_matmul(device, wt, Tensor.from_data(x), Tensor.from_data(bias), False, True, to)
             want = oracle.matmul_ref(buf, odt, (S, N, K), x, oracle.F16, x.shape, bias, False, True, to)
             check(oracle, got, want, DType.F16, (kind, S, N, K, M, to))
+
+
+@pytest.mark.parametrize("rows_w,rows_x", [(1280, 768), (1280, 1408), (2560, 640)], ids=["8x6", "8x11", "16x5"])
+@pytest.mark.parametrize("quant", [False, True], ids=["f16", "q8_0h"])
+def test_large_tile_panel_order(device, oracle, rows_w, rows_x, quant):
+    """Large-tile NT GEMMs with whole weight row blocks per XCD and more than four activation column blocks walk
+    their tiles in panels of four column blocks (a narrower last panel included): every output tile must be
+    written exactly once.  The output of each 160 x 128 tile depends on its position (distinct rows of both
+    operands), so a tile computed twice or never shows against the oracle."""
+    rng = np.random.default_rng(rows_w + rows_x)
+    K = 256
+    w = (rng.standard_normal((rows_w, K)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((1, rows_x, K)).astype(np.float16)
+    bias = rng.standard_normal(rows_w).astype(np.float16)
+    if quant:
+        buf = oracle.make_q8_0h(w)
+        lhs = Tensor.from_quantized(buf, DType.Q8_0H, (rows_w, K))
+        want = oracle.matmul_ref(buf, oracle.Q8_0H, (rows_w, K), x, oracle.F16, x.shape, bias, False, True, True)
+    else:
+        wh = w.astype(np.float16)
+        lhs = Tensor.from_data(wh)
+        want = oracle.matmul_ref(wh, oracle.F16, wh.shape, x, oracle.F16, x.shape, bias, False, True, True)
+    got = gpu_matmul(device, lhs, Tensor.from_data(x), Tensor.from_data(bias), False, True, True)
+    assert got.shape == (1, rows_x, rows_w)
+    assert oracle.max_rel_err(got, want) <= 2e-2
