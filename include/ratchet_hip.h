@@ -174,7 +174,12 @@ RT_API const char *rt_kernel_string(int32_t kernel_kind);
 /* ---- device context and buffers ------------------------------------------ */
 
 /* Replaces: Device::request_device(DeviceRequest::GPU) / WgpuDevice::new
- * (crates/ratchet-core/src/device.rs:37-56, gpu/device.rs:62-140). */
+ * (crates/ratchet-core/src/device.rs:37-56, gpu/device.rs:62-140).
+ * Checked mode: when the environment variable RATCHET_CHECKED (the reference's switch for its checked
+ * shader builds, gpu/pools/kernel_module_pool.rs:62-67) is set to anything but "0" at this call, every
+ * matmul enqueue on the context first looks up the device allocation behind each pointer and fails with
+ * RT_ERR_INVALID_ARG when it holds fewer bytes than the descriptor implies.  A query per pointer and
+ * call: for debugging, not for serving. */
 RT_API rt_status rt_ctx_create(int32_t device_ordinal, rt_ctx **ctx);
 RT_API rt_status rt_ctx_destroy(rt_ctx *ctx);
 

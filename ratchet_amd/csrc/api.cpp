@@ -3,6 +3,7 @@
 // host: a missing device is an error, never a fallback.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -33,6 +34,11 @@ struct rt_ctx {
     int last_hip = 0;
     void *static_scratch = nullptr;   // device address of `scratch` on this context's GPU
     hipError_t static_scratch_err = hipSuccess;
+    // Checked mode (the environment variable RATCHET_CHECKED, as in the reference's
+    // gpu/pools/kernel_module_pool.rs:62-67, read when the context is created): before a matmul is
+    // enqueued every operand's device allocation is looked up and must hold the bytes the descriptor
+    // implies.  Costs a runtime query per pointer and call; off by default.
+    bool checked = false;
 };
 
 namespace {
@@ -47,6 +53,29 @@ rt_status fail(rt_ctx *ctx, rt_status st, const std::string &msg, hipError_t her
         }
     }
     return st;
+}
+
+// Checked mode: `ptr` must lie in a device allocation that extends at least `need` bytes past it.
+rt_status check_extent(rt_ctx *ctx, const void *ptr, uint64_t need, const char *what) {
+    if (!ptr || need == 0) return RT_OK;
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    const hipError_t e = hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(ctx, RT_ERR_INVALID_ARG, std::string("checked: ") + what + " is not a device allocation");
+    }
+    const uint64_t off = (uint64_t)((const uint8_t *)ptr - (const uint8_t *)base);
+    if (off > size || size - off < need)
+        return fail(ctx, RT_ERR_INVALID_ARG, std::string("checked: ") + what + " holds " + std::to_string(size - off) +
+                                                 " bytes from the pointer on, the descriptor needs " + std::to_string(need));
+    return RT_OK;
+}
+
+uint64_t shape_numel(const int64_t *shape, int32_t rank) {
+    uint64_t n = 1;
+    for (int32_t i = 0; i < rank; i++) n *= (uint64_t)shape[i];
+    return n;
 }
 
 rt_status hip_fail(rt_ctx *ctx, const char *what, hipError_t e) {
@@ -176,6 +205,7 @@ rt_status rt_ctx_create(int32_t device_ordinal, rt_ctx **ctx) {
         if (c->static_scratch_err == hipSuccess) c->static_scratch = ptr;
         else (void)hipGetLastError();
     }
+    if (const char *env = std::getenv("RATCHET_CHECKED")) c->checked = env[0] != '\0' && !(env[0] == '0' && env[1] == '\0');
     *ctx = c;
     return RT_OK;
     RT_GUARD_END(nullptr)
@@ -283,6 +313,19 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
     const void *A = p.swapped ? rhs : lhs, *B = p.swapped ? lhs : rhs;
     DeviceGuard dg(ctx->dev.ordinal);
     if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
+    if (ctx->checked) {
+        uint64_t nl = 0, nr = 0, nb = 0;
+        if (rt_tensor_nbytes(desc->lhs_dt, shape_numel(desc->lhs_shape, desc->lhs_rank), &nl) != RT_OK ||
+            rt_tensor_nbytes(desc->rhs_dt, shape_numel(desc->rhs_shape, desc->rhs_rank), &nr) != RT_OK ||
+            (desc->has_bias && rt_tensor_nbytes(desc->bias_dt, shape_numel(desc->bias_shape, desc->bias_rank), &nb) != RT_OK))
+            return fail(ctx, RT_ERR_INVALID_ARG, "checked: operand sizes");
+        const uint64_t no = (uint64_t)p.stacks * (uint64_t)p.M * (uint64_t)p.N * (p.act_dt == RT_F16 ? 2u : 4u);
+        if ((st = check_extent(ctx, lhs, nl, "lhs")) != RT_OK || (st = check_extent(ctx, rhs, nr, "rhs")) != RT_OK ||
+            (st = check_extent(ctx, desc->has_bias ? bias : nullptr, nb, "bias")) != RT_OK ||
+            (st = check_extent(ctx, out, no, "out")) != RT_OK ||
+            (st = check_extent(ctx, p.workspace, p.workspace_bytes, "workspace")) != RT_OK)
+            return st;
+    }
     hipError_t e = hipErrorNotSupported;
     if (p.kernel == RT_KERNEL_GEMV_Q8 || p.kernel == RT_KERNEL_GEMV_Q4K || p.kernel == RT_KERNEL_GEMV_FLOAT)
         e = rt::launch_gemv(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);

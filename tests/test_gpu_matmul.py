@@ -770,3 +770,56 @@ def test_large_tile_panel_order(device, oracle, rows_w, rows_x, quant):
     got = gpu_matmul(device, lhs, Tensor.from_data(x), Tensor.from_data(bias), False, True, True)
     assert got.shape == (1, rows_x, rows_w)
     assert oracle.max_rel_err(got, want) <= 2e-2
+
+
+def test_checked_mode_refuses_short_buffers(device, oracle, monkeypatch):
+    """RATCHET_CHECKED (read by rt_ctx_create): an operand or output allocation smaller than the descriptor
+    implies is refused with a status before anything is launched; exact allocations pass and compute."""
+    import ctypes
+
+    from ratchet_amd import _ffi
+    L = _ffi.lib()
+    monkeypatch.setenv("RATCHET_CHECKED", "1")
+    ctx = ctypes.c_void_p()
+    assert L.rt_ctx_create(device.ordinal, ctypes.byref(ctx)) == _ffi.RT_OK
+    try:
+        N, M, K = 256, 64, 512
+        rng = np.random.default_rng(77)
+        w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+        buf = oracle.make_q8_0h(w)
+        x = rng.standard_normal((1, M, K)).astype(np.float16)
+        desc = _ffi.make_desc(_ffi.RT_Q8_0H, (N, K), _ffi.RT_F16, (1, M, K), False, True, True)
+
+        def alloc(nbytes, data=None):
+            p = ctypes.c_void_p()
+            assert L.rt_buf_alloc(ctx, nbytes, ctypes.byref(p)) == _ffi.RT_OK
+            if data is not None:
+                host = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+                assert L.rt_buf_upload(ctx, p, host.ctypes.data_as(ctypes.c_void_p), host.size, None) == _ffi.RT_OK
+                assert L.rt_sync(ctx, None) == _ffi.RT_OK
+            return p
+
+        dw, dx = alloc(buf.nbytes, buf), alloc(x.nbytes, x)
+        out_ok, out_short = alloc(M * N * 2), alloc(M * N * 2 - 256)
+        w_short = alloc(buf.nbytes - 4096)
+        bufs = [dw, dx, out_ok, out_short, w_short]
+        stream = ctypes.c_void_p(0)
+        st = L.rt_matmul_enqueue(ctx, ctypes.byref(desc), dw, dx, None, out_short, stream)
+        assert st == _ffi.RT_ERR_INVALID_ARG and b"out holds" in L.rt_last_error(ctx)
+        st = L.rt_matmul_enqueue(ctx, ctypes.byref(desc), w_short, dx, None, out_ok, stream)
+        assert st == _ffi.RT_ERR_INVALID_ARG and b"lhs holds" in L.rt_last_error(ctx)
+        # a pointer into the middle of an allocation counts from there
+        st = L.rt_matmul_enqueue(ctx, ctypes.byref(desc), dw, dx, None, ctypes.c_void_p(out_ok.value + 512), stream)
+        assert st == _ffi.RT_ERR_INVALID_ARG
+        st = L.rt_matmul_enqueue(ctx, ctypes.byref(desc), dw, dx, None, out_ok, stream)
+        assert st == _ffi.RT_OK, L.rt_last_error(ctx)
+        assert L.rt_sync(ctx, stream) == _ffi.RT_OK
+        got = np.empty((1, M, N), dtype=np.float16)
+        assert L.rt_buf_download(ctx, got.ctypes.data_as(ctypes.c_void_p), out_ok, got.nbytes, None) == _ffi.RT_OK
+        assert L.rt_sync(ctx, None) == _ffi.RT_OK
+        want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, None, False, True, True)
+        assert oracle.max_rel_err(got, want) <= 2e-2
+        for b in bufs:
+            L.rt_buf_free(ctx, b)
+    finally:
+        L.rt_ctx_destroy(ctx)
