@@ -322,10 +322,13 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     l_run += __shfl_xor(l_run, 32, kWave);
     if (g.splits > 1) {
         // this workgroup saw only its share of the keys: hand (m, l, O) of every row to the merge kernel
+        // (rows past q_len are never merged: a decode step has one live row of 64)
         float *pr = g.partial + ((((size_t)blockIdx.y * gridDim.x + blockIdx.x) * g.splits + split) * AT_BQ + 16 * qt + fr) * (4 + DP);
-        if (fg == 0) pr[0] = m_run, pr[1] = l_run;
+        if (qrow < g.q_len) {
+            if (fg == 0) pr[0] = m_run, pr[1] = l_run;
 #pragma unroll
-        for (int d = 0; d < DT; d++) *(float4_t *)(pr + 4 + 16 * d + 4 * fg) = acc[d];
+            for (int d = 0; d < DT; d++) *(float4_t *)(pr + 4 + 16 * d + 4 * fg) = acc[d];
+        }
         return;
     }
     const float inv = 1.f / l_run; // no visible key: 0 / 0 = NaN, what the unfused sequence yields
