@@ -515,7 +515,10 @@ def test_f16_untransposed_narrow_rhs(device, oracle):
     """`lhs.matmul(rhs)` with an N-contiguous rhs of at most 128 columns (the attention P.V form):
     row counts off the 32-row grouping, K off the 64 tile, every N tile count, stacks, broadcast, bias."""
     shapes = [(2, 64, 64, 80), (1, 100, 72, 8), (3, 257, 200, 128), (1, 512, 512, 80), (1, 65, 8, 16),
-              (2, 96, 136, 48), (1, 1000, 320, 104)]
+              (2, 96, 136, 48), (1, 1000, 320, 104),
+              # more K tiles than are in flight at once (whole and ragged), and stack counts that take the
+              # XCD-aware workgroup order with whole and ragged row blocks
+              (1, 128, 1024, 80), (2, 70, 1160, 40), (8, 100, 72, 24), (16, 128, 576, 64)]
     for i, (S, M, K, N) in enumerate(shapes):
         rng = np.random.default_rng(800 + i)
         a = rng.standard_normal((S, M, K)).astype(np.float16)
