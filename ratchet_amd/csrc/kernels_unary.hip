@@ -7,23 +7,39 @@
 
 namespace rt {
 
+// A thread takes UNARY_U vectors of 16 bytes a workgroup-width apart and requests them all before it
+// evaluates the first: with one vector per thread the launch is a single trip to memory per wavefront
+// with nothing else in flight.  Loads and stores are non-temporal: every byte is touched once.
+constexpr int UNARY_U = 4;
+
 template <typename T, int ACT>
 __global__ __launch_bounds__(256) void unary_kernel(const T *src, T *dst, uint64_t numel) {
     constexpr int EV = 16 / sizeof(T);
     const uint64_t nvec = numel / EV;
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    for (uint64_t v = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
-        const uint4_t raw = ((const uint4_t *)src)[v];
-        if constexpr (sizeof(T) == 2) {
-            half8_t h = __builtin_bit_cast(half8_t, raw);
+    const uint64_t stride = (uint64_t)gridDim.x * (256 * UNARY_U);
+    for (uint64_t v0 = (uint64_t)blockIdx.x * (256 * UNARY_U) + threadIdx.x; v0 < nvec; v0 += stride) {
+        uint4_t raw[UNARY_U];
 #pragma unroll
-            for (int e = 0; e < 8; e++) h[e] = (half_t)rt_act((float)h[e], ACT);
-            ((uint4_t *)dst)[v] = __builtin_bit_cast(uint4_t, h);
-        } else {
-            float4_t f = __builtin_bit_cast(float4_t, raw);
+        for (int u = 0; u < UNARY_U; u++) {
+            const uint64_t v = v0 + 256u * u;
+            raw[u] = __builtin_nontemporal_load((const uint4_t *)src + (v < nvec ? v : nvec - 1)); // past the end: a valid vector, not stored
+        }
 #pragma unroll
-            for (int e = 0; e < 4; e++) f[e] = rt_act(f[e], ACT);
-            ((uint4_t *)dst)[v] = __builtin_bit_cast(uint4_t, f);
+        for (int u = 0; u < UNARY_U; u++) {
+            const uint64_t v = v0 + 256u * u;
+            uint4_t res;
+            if constexpr (sizeof(T) == 2) {
+                half8_t h = __builtin_bit_cast(half8_t, raw[u]);
+#pragma unroll
+                for (int e = 0; e < 8; e++) h[e] = (half_t)rt_act((float)h[e], ACT);
+                res = __builtin_bit_cast(uint4_t, h);
+            } else {
+                float4_t f = __builtin_bit_cast(float4_t, raw[u]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) f[e] = rt_act(f[e], ACT);
+                res = __builtin_bit_cast(uint4_t, f);
+            }
+            if (v < nvec) __builtin_nontemporal_store(res, (uint4_t *)dst + v);
         }
     }
     // the elements past the last whole vector
@@ -34,19 +50,42 @@ __global__ __launch_bounds__(256) void unary_kernel(const T *src, T *dst, uint64
 
 template <typename S, typename D>
 __global__ __launch_bounds__(256) void cast_kernel(const S *src, D *dst, uint64_t numel) {
-    // 8 elements per thread: 32 bytes of f32 <-> 16 bytes of f16
+    // 8 elements per vector: 32 bytes of f32 <-> 16 bytes of f16; UNARY_U vectors per thread, all requested
+    // before the first is converted, non-temporal both ways
     const uint64_t nvec = numel / 8;
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    for (uint64_t v = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
+    const uint64_t stride = (uint64_t)gridDim.x * (256 * UNARY_U);
+    for (uint64_t v0 = (uint64_t)blockIdx.x * (256 * UNARY_U) + threadIdx.x; v0 < nvec; v0 += stride) {
         if constexpr (sizeof(S) == 4) {
-            const float4_t a = ((const float4_t *)src)[2 * v], b = ((const float4_t *)src)[2 * v + 1];
-            const half8_t h = {(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3],
-                               (half_t)b[0], (half_t)b[1], (half_t)b[2], (half_t)b[3]};
-            ((uint4_t *)dst)[v] = __builtin_bit_cast(uint4_t, h);
+            float4_t a[UNARY_U], b[UNARY_U];
+#pragma unroll
+            for (int u = 0; u < UNARY_U; u++) {
+                const uint64_t v = v0 + 256u * u < nvec ? v0 + 256u * u : nvec - 1; // past the end: a valid vector, not stored
+                a[u] = __builtin_nontemporal_load((const float4_t *)src + 2 * v);
+                b[u] = __builtin_nontemporal_load((const float4_t *)src + 2 * v + 1);
+            }
+#pragma unroll
+            for (int u = 0; u < UNARY_U; u++) {
+                const uint64_t v = v0 + 256u * u;
+                const half8_t h = {(half_t)a[u][0], (half_t)a[u][1], (half_t)a[u][2], (half_t)a[u][3],
+                                   (half_t)b[u][0], (half_t)b[u][1], (half_t)b[u][2], (half_t)b[u][3]};
+                if (v < nvec) __builtin_nontemporal_store(__builtin_bit_cast(uint4_t, h), (uint4_t *)dst + v);
+            }
         } else {
-            const half8_t h = __builtin_bit_cast(half8_t, ((const uint4_t *)src)[v]);
-            ((float4_t *)dst)[2 * v] = float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
-            ((float4_t *)dst)[2 * v + 1] = float4_t{(float)h[4], (float)h[5], (float)h[6], (float)h[7]};
+            uint4_t raw[UNARY_U];
+#pragma unroll
+            for (int u = 0; u < UNARY_U; u++) {
+                const uint64_t v = v0 + 256u * u < nvec ? v0 + 256u * u : nvec - 1;
+                raw[u] = __builtin_nontemporal_load((const uint4_t *)src + v);
+            }
+#pragma unroll
+            for (int u = 0; u < UNARY_U; u++) {
+                const uint64_t v = v0 + 256u * u;
+                const half8_t h = __builtin_bit_cast(half8_t, raw[u]);
+                if (v < nvec) {
+                    __builtin_nontemporal_store(float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]}, (float4_t *)dst + 2 * v);
+                    __builtin_nontemporal_store(float4_t{(float)h[4], (float)h[5], (float)h[6], (float)h[7]}, (float4_t *)dst + 2 * v + 1);
+                }
+            }
         }
     }
     const uint64_t i = nvec * 8 + (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -59,7 +98,7 @@ static unsigned grid_for(uint64_t nvec, const unsigned cap = 256u * 32u) {
 }
 
 template <typename T> static hipError_t launch_unary_t(int act, const void *src, void *dst, uint64_t numel, hipStream_t st) {
-    const unsigned grid = grid_for(numel / (16 / sizeof(T)));
+    const unsigned grid = grid_for((numel / (16 / sizeof(T)) + UNARY_U - 1) / UNARY_U);
     if (act == RT_ACT_GELU)
         hipLaunchKernelGGL((unary_kernel<T, RT_ACT_GELU>), dim3(grid), dim3(256), 0, st, (const T *)src, (T *)dst, numel);
     else
@@ -76,7 +115,7 @@ hipError_t launch_unary(int act, int dtype, const void *src, void *dst, uint64_t
 
 hipError_t launch_cast(int src_dtype, int dst_dtype, const void *src, void *dst, uint64_t numel, hipStream_t stream) {
     if (numel == 0) return hipSuccess;
-    const unsigned grid = grid_for(numel / 8);
+    const unsigned grid = grid_for((numel / 8 + UNARY_U - 1) / UNARY_U);
     if (src_dtype == RT_F32 && dst_dtype == RT_F16)
         hipLaunchKernelGGL((cast_kernel<float, half_t>), dim3(grid), dim3(256), 0, stream, (const float *)src, (half_t *)dst, numel);
     else if (src_dtype == RT_F16 && dst_dtype == RT_F32)
