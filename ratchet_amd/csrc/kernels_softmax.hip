@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(T *x, int64_t rows, i
     for (int i = 0; i < VPL; i++) {
         const int v = lane + 64 * i;
         uint4_t raw = {0u, 0u, 0u, 0u};
-        if (v < nvec) raw = p[v];
+        if (v < nvec) raw = __builtin_nontemporal_load(p + v); // read once, written once: nothing to keep in the caches
 #pragma unroll
         for (int e = 0; e < EV; e++) {
             f[i][e] = v < nvec ? SoftmaxVec<T>::get(raw, e) : ninf;
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(T *x, int64_t rows, i
 #pragma unroll
     for (int i = 0; i < VPL; i++) {
         const int v = lane + 64 * i;
-        if (v < nvec) p[v] = SoftmaxVec<T>::make([&](int e) { return f[i][e] / s; });
+        if (v < nvec) __builtin_nontemporal_store(SoftmaxVec<T>::make([&](int e) { return f[i][e] / s; }), p + v);
     }
 }
 
