@@ -201,7 +201,7 @@ __global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr_kernel(GemmNnArgs g) {
     for (int v = lane; v < 16 * nvec; v += 64) {
         const int il = v / nvec, c = v - il * nvec;
         const int64_t i = i0 + rw * 16 + il;
-        if (i < g.M) *(uint4_t *)(out + i * g.o_is + 8 * c) = *(const uint4_t *)(es + il * EROW + 8 * c);
+        if (i < g.M) __builtin_nontemporal_store(*(const uint4_t *)(es + il * EROW + 8 * c), (uint4_t *)(out + i * g.o_is + 8 * c));
     }
 }
 

@@ -150,7 +150,7 @@ __device__ __forceinline__ void nt_epilogue(const GemmNtArgs &g, float4_t (&acc)
             const int64_t j = j0 + wj * WN + jl, i = i0 + wi * WM + 8 * c;
             if (j < g.N) {
                 if (i + 8 <= g.M) {
-                    *(uint4_t *)(out + j * g.o_js + i) = *(const uint4_t *)(es + jl * EROW + 8 * c);
+                    __builtin_nontemporal_store(*(const uint4_t *)(es + jl * EROW + 8 * c), (uint4_t *)(out + j * g.o_js + i)); // written once, not read back here
                 } else {
                     for (int e = 0; e < 8; e++)
                         if (i + e < g.M) out[j * g.o_js + i + e] = es[jl * EROW + 8 * c + e];
