@@ -42,7 +42,10 @@ constexpr int F32_LDA = F32_BK + 4;
 
 // B_KCONT: B's K axis is the contiguous one (its tile is [col][k], like A's); otherwise its
 // column axis is (tile [k][col]).
-template <int BM, int BN, bool B_KCONT, bool KTAIL>
+// OJ: the output's column axis is the contiguous one (row-major C).  The MFMA's operands are then
+// exchanged, which transposes what a lane holds: four consecutive columns of one row instead of four
+// consecutive rows of one column, so the epilogue writes 16 bytes per lane either way.
+template <int BM, int BN, bool B_KCONT, bool KTAIL, bool OJ>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
     static_assert(WM % 16 == 0 && WN % 16 == 0, "a wavefront's share must split into 16 x 16 MFMA tiles");
@@ -168,7 +171,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
                 for (int a = 0; a < TM; a++)
 #pragma unroll
                     for (int b = 0; b < TN; b++)
-                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[kk & 1][a], fb[kk & 1][b], acc[a][b], 0, 0, 0);
+                        acc[a][b] = OJ ? __builtin_amdgcn_mfma_f32_16x16x4f32(fb[kk & 1][b], fa[kk & 1][a], acc[a][b], 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_f32_16x16x4f32(fa[kk & 1][a], fb[kk & 1][b], acc[a][b], 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -186,18 +190,46 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
         if (kt + 1 < nk) k_tile(kt + 1, r1, r0);
     }
 
-    // acc[a][b][r] is C[i0 + wi WM + 16 a + 4 fq + r][j0 + wj WN + 16 b + fr]
     float *out = g.out + s * g.o_bs;
     const int64_t iw = i0 + wi * WM, jw = j0 + wj * WN; // this wavefront's corner
+    if constexpr (OJ) {
+        // acc[a][b][r] is C[iw + 16 a + fr][jw + 16 b + 4 fq + r]: 16 bytes per lane along a row (non-temporal:
+        // the output is written once), 64 contiguous bytes per row and instruction
+        rt_with_act(g.act, [&](auto has_act) {
+#pragma unroll
+            for (int a = 0; a < TM; a++) {
+                const int64_t i = iw + 16 * a + fr;
+                if (i >= g.M) continue;
+#pragma unroll
+                for (int b = 0; b < TN; b++) {
+                    const int64_t j = jw + 16 * b + 4 * fq;
+                    if (j >= g.N) continue; // N % 4 == 0: a group of four is inside or outside as a whole
+                    float4_t v = acc[a][b];
+                    if (g.has_bias) {
+                        if (g.bias_on_rows) {
+                            const float bi = g.bias[i];
+                            v += float4_t{bi, bi, bi, bi};
+                        } else {
+                            v += *(const float4_t *)(g.bias + j);
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; r++) v[r] = rt_act_k<decltype(has_act)::value>(v[r]);
+                    __builtin_nontemporal_store(v, (float4_t *)(out + i * g.o_is + j));
+                }
+            }
+        });
+        return;
+    }
+    // acc[a][b][r] is C[iw + 16 a + 4 fq + r][jw + 16 b + fr]
     auto value = [&](auto has_act, int a, int b, int r) {
         float x = acc[a][b][r];
         if (g.has_bias) x += g.bias[g.bias_on_rows ? min(iw + 16 * a + 4 * fq + r, g.M - 1) : min(jw + 16 * b + fr, g.N - 1)];
         x = rt_act_k<decltype(has_act)::value>(x);
         return x;
     };
-    // Straight from the accumulators: a store instruction covers 64 contiguous bytes of four rows
-    // (row-major output), or 16 bytes per lane along the rows (o_is == 1).  Staging the sub-tile
-    // through LDS for 128-bit stores over whole runs measured 1 us slower at the Whisper shape.
+    // Straight from the accumulators: 16 bytes per lane along the rows (o_is == 1), or scalar stores.
+    // Staging the sub-tile through LDS for 128-bit stores over whole runs measured 1 us slower at the Whisper shape.
     rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
         for (int a = 0; a < TM; a++)
@@ -217,15 +249,22 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     });
 }
 
-template <int BM, int BN, bool B_KCONT, bool KTAIL>
-static hipError_t launch_f32_kt(const GemmF32Args &g, int64_t stacks, hipStream_t st) {
+template <int BM, int BN, bool B_KCONT, bool KTAIL, bool OJ>
+static hipError_t launch_f32_oj(const GemmF32Args &g, int64_t stacks, hipStream_t st) {
     constexpr int LDB = B_KCONT ? F32_LDA : BN + 16;
     constexpr size_t lds = (size_t)2 * (BM * F32_LDA + (B_KCONT ? BN * F32_LDA : F32_BK * LDB)) * sizeof(float);
-    if (const hipError_t e = ensure_lds_limit<&gemm_f32_kernel<BM, BN, B_KCONT, KTAIL>>(); e != hipSuccess) return e;
+    if (const hipError_t e = ensure_lds_limit<&gemm_f32_kernel<BM, BN, B_KCONT, KTAIL, OJ>>(); e != hipSuccess) return e;
     const int64_t tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     if (tiles > 0x7fffffff) return hipErrorNotSupported;
-    hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, B_KCONT, KTAIL>), dim3((unsigned)tiles, (unsigned)stacks), dim3(256), lds, st, g);
+    hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, B_KCONT, KTAIL, OJ>), dim3((unsigned)tiles, (unsigned)stacks), dim3(256), lds, st, g);
     return hipGetLastError();
+}
+
+template <int BM, int BN, bool B_KCONT, bool KTAIL>
+static hipError_t launch_f32_kt(const GemmF32Args &g, int64_t stacks, hipStream_t st) {
+    // row-major output with 16-byte aligned rows and N % 4 == 0 (bias along the columns read as vectors)
+    const bool oj = g.o_js == 1 && g.N % 4 == 0 && g.o_is % 4 == 0 && g.o_bs % 4 == 0 && (!g.has_bias || g.bias_on_rows || ((uintptr_t)g.bias & 15u) == 0);
+    return oj ? launch_f32_oj<BM, BN, B_KCONT, KTAIL, true>(g, stacks, st) : launch_f32_oj<BM, BN, B_KCONT, KTAIL, false>(g, stacks, st);
 }
 
 template <int BM, int BN, bool B_KCONT>
