@@ -628,6 +628,8 @@ def main():
                     help="run only the two C4 GEMM workloads (f16 and Q8_0H weights) and print their lines; for profiling")
     ap.add_argument("--c3-only", action="store_true",
                     help="run only the attention products of configs[2] and print their lines; for profiling")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="run only the fused attention workloads (prefill, causal prefill, one decode step); for profiling")
     ap.add_argument("--q4k-only", action="store_true",
                     help="run only the Q4_K prefill workload (C5 at 256 rows) and print its line; for profiling")
     ap.add_argument("--read-calibration", action="store_true",
@@ -667,6 +669,11 @@ def main():
 
     if args.c3_only:
         for g in c3_products(r, O):
+            print(json.dumps(g))
+        return 0
+
+    if args.attention_only:
+        for g in bench_attention(r, O):
             print(json.dumps(g))
         return 0
 

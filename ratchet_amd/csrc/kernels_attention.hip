@@ -388,6 +388,158 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs g) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Decoding: one query row per head against a long cache.  The tiled kernel above would spend a 64-row
+// query block and its matrix instructions on one live row; this one is a stream over the keys and
+// values, like the GEMV of a decode step.  A workgroup of four wavefronts takes 128 consecutive keys
+// of one head: 16 lanes share a key (lane `seg` holds dimensions 8 seg .. + 7: 16 bytes of the key and
+// 16 of the value, lanes past head_dim / 8 idle), so a wavefront's load covers four whole keys, and
+// all 8 + 8 loads of a lane are requested before the first is used.  The score is 4 v_dot2_f32_f16
+// and four DPP additions inside the 16-lane row; the softmax of the 128 keys is local (maximum and
+// sum through LDS), the probabilities stay f32, and the 16 key slots' shares of the output meet in
+// LDS.  Every workgroup writes (maximum, sum, unnormalised output) of its keys; a second small
+// kernel merges the splits of a head exactly as the tiled kernel's merge does.
+// ---------------------------------------------------------------------------------------------
+constexpr int AD_THREADS = 256, AD_L = 8, AD_KEYS = 16 * AD_L; // key slots per load x loads = keys per workgroup
+constexpr int AD_PSTRIDE = 4 + 128;                            // floats per (head, split) in the workspace
+
+template <int CTRL> __device__ __forceinline__ float ad_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// sum over the 16 lanes of a row, left in all of them
+__device__ __forceinline__ float ad_row_sum(float v) {
+    v += ad_dpp<0x128>(v); // row_ror:8
+    v += ad_dpp<0x124>(v); // row_ror:4
+    v += ad_dpp<0x122>(v); // row_ror:2
+    v += ad_dpp<0x121>(v); // row_ror:1
+    return v;
+}
+__device__ __forceinline__ float ad_wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+__global__ __launch_bounds__(AD_THREADS) void attention_decode_kernel(AttnArgs g) {
+    __shared__ float sm[4], sl[4];
+    __shared__ __attribute__((aligned(16))) float so[16][16][8]; // [key slot][seg][8 dimensions]
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int seg = lane & 15, slot = wave * 4 + (lane >> 4);
+    const int ns = g.D >> 3;
+    const int segc = min(seg, ns - 1); // idle lanes repeat the last live lane's addresses (no extra traffic) and contribute zeros
+    const int split = blockIdx.x, bh = blockIdx.y, b = bh / g.heads, h = bh - b * g.heads;
+    const half_t *Q = g.Q + b * g.q_bs + h * g.q_hs;
+    const half_t *K = g.K + b * g.k_bs + h * g.k_hs;
+    const half_t *V = g.V + b * g.v_bs + h * g.v_hs;
+    const uint4_t zero4 = {0u, 0u, 0u, 0u};
+    const int key0 = split * AD_KEYS + slot;
+
+    uint4_t kr[AD_L], vr[AD_L];
+#pragma unroll
+    for (int i = 0; i < AD_L; i++) {
+        const uint32_t kc = (uint32_t)min(key0 + 16 * i, g.kv_len - 1); // past the last key: a valid one, masked below
+        kr[i] = __builtin_nontemporal_load((const uint4_t *)(K + (kc * (uint32_t)g.k_rs + 8u * segc)));
+    }
+#pragma unroll
+    for (int i = 0; i < AD_L; i++) {
+        const uint32_t kc = (uint32_t)min(key0 + 16 * i, g.kv_len - 1);
+        vr[i] = __builtin_nontemporal_load((const uint4_t *)(V + (kc * (uint32_t)g.v_rs + 8u * segc)));
+    }
+    uint4_t qv = *(const uint4_t *)(Q + 8 * segc);
+    if (seg >= ns) qv = zero4;
+
+    // scores in base-2 units, the same in all 16 lanes of a key
+    float sc[AD_L], m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < AD_L; i++) {
+        float p = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t qa = qv[e], ka = kr[i][e];
+            p = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qa), __builtin_bit_cast(half2_t, ka), p, false);
+        }
+        p = ad_row_sum(p);
+        sc[i] = key0 + 16 * i < g.kv_len ? p * g.scale_log2e : -INFINITY;
+        m = fmaxf(m, sc[i]);
+    }
+    m = ad_wave_max(m);
+    if (lane == 0) sm[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+    const float m_use = m == -INFINITY ? 0.f : m; // no visible key here: every weight is exp2(-inf) = 0
+
+    // probabilities (f32) and this lane's 8 dimensions of sum_k p_k v_k over its key slot
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, l = 0.f;
+#pragma unroll
+    for (int i = 0; i < AD_L; i++) {
+        const float p = __builtin_amdgcn_exp2f(sc[i] - m_use);
+        l += p;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t va = vr[i][e];
+            const half2_t v2 = __builtin_bit_cast(half2_t, va);
+            acc[2 * e] = fmaf(p, (float)v2[0], acc[2 * e]);
+            acc[2 * e + 1] = fmaf(p, (float)v2[1], acc[2 * e + 1]);
+        }
+    }
+    // a key's probability sits in all 16 lanes of its row: the wavefront's sum counts it 16 times
+    l = wave_sum(l) * (1.f / 16.f);
+    if (lane == 0) sl[wave] = l;
+    *(float4_t *)&so[slot][seg][0] = float4_t{acc[0], acc[1], acc[2], acc[3]};
+    *(float4_t *)&so[slot][seg][4] = float4_t{acc[4], acc[5], acc[6], acc[7]};
+    __syncthreads();
+    float *pr = g.partial + ((size_t)bh * g.splits + split) * AD_PSTRIDE;
+    if (t == 0) pr[0] = m, pr[1] = (sl[0] + sl[1]) + (sl[2] + sl[3]);
+    if (t < g.D) {
+        float o = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) o += so[k][t >> 3][t & 7];
+        pr[4 + t] = o;
+    }
+}
+
+// One workgroup per head: thread d combines dimension d of the head's splits.
+__global__ __launch_bounds__(128) void attention_decode_merge_kernel(AttnArgs g) {
+    const int bh = blockIdx.x, b = bh / g.heads, h = bh - b * g.heads, d = threadIdx.x;
+    const float *base = g.partial + (size_t)bh * g.splits * AD_PSTRIDE;
+    // running (maximum, sum, output), sixteen splits' values requested at a time: the partial results come
+    // from other XCDs' workgroups, so every round of loads is a trip to memory, and a cache of 2048 keys is one round
+    float m = -INFINITY, l = 0.f, o = 0.f;
+    const int dc = min(d, g.D - 1);
+    for (int s0 = 0; s0 < g.splits; s0 += 16) {
+        float ms[16], ls[16], os[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const float *ps = base + (size_t)min(s0 + u, g.splits - 1) * AD_PSTRIDE; // past the last split: re-read it, skipped below
+            ms[u] = ps[0], ls[u] = ps[1], os[u] = ps[4 + dc];
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            if (s0 + u < g.splits) {
+                const float m_new = fmaxf(m, ms[u]);
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                const float a = __builtin_amdgcn_exp2f(m - m_use), w = __builtin_amdgcn_exp2f(ms[u] - m_use);
+                l = l * a + ls[u] * w;
+                o = o * a + os[u] * w;
+                m = m_new;
+            }
+        }
+    }
+    if (d < g.D) g.O[b * g.o_bs + h * g.o_hs + d] = (half_t)(o / l); // no visible key anywhere: 0 / 0 = NaN, as in the single pass
+}
+
+// splits of the decode kernel for this problem, or 0 when it does not apply: one query row (the causal rule
+// then hides nothing), a cache long enough to be worth two kernels; a launch with a mask tensor stays tiled
+static int attention_decode_splits(const rt_attention_desc &d) {
+    if (d.q_len != 1 || d.kv_len < 256 || d.head_dim % 8 != 0 || d.head_dim > 128) return 0;
+    return (d.kv_len + AD_KEYS - 1) / AD_KEYS;
+}
+static uint64_t attention_decode_workspace_bytes(const rt_attention_desc &d) {
+    return (uint64_t)d.batch * d.heads * attention_decode_splits(d) * AD_PSTRIDE * sizeof(float);
+}
+
 template <int DP, bool MASK> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
     constexpr int STAGES = DP <= 96 ? 4 : 3;
     // the ring of packed key + value blocks; the merge of the key halves reuses it
@@ -429,9 +581,9 @@ int attention_splits(const rt_attention_desc &d) {
 // bytes of workspace a split launch of this problem needs (0: it runs in one pass)
 uint64_t attention_workspace_bytes(const rt_attention_desc &d) {
     const int s = attention_splits(d);
-    if (s <= 1) return 0;
     const uint64_t qb = (uint64_t)((d.q_len + AT_BQ - 1) / AT_BQ);
-    return qb * (uint64_t)d.batch * d.heads * s * AT_BQ * (4 + attention_dp(d.head_dim)) * sizeof(float);
+    const uint64_t tiled = s <= 1 ? 0 : qb * (uint64_t)d.batch * d.heads * s * AT_BQ * (4 + attention_dp(d.head_dim)) * sizeof(float);
+    return std::max(tiled, attention_decode_workspace_bytes(d)); // whichever of the two split paths the launch takes
 }
 
 // f16 tensors, head_dim a multiple of 8 up to 128, rows 16-byte aligned.  `workspace` may be null
@@ -456,6 +608,15 @@ hipError_t launch_attention(const rt_attention_desc &d, const void *q, const voi
     // 32-bit element offsets inside one head's keys and values
     if ((int64_t)d.kv_len * g.k_rs >= (int64_t(1) << 31) || (int64_t)d.kv_len * g.v_rs >= (int64_t(1) << 31))
         return hipErrorNotSupported;
+    // one query against a long cache: the streaming kernel, when the caller gave the workspace for it
+    if (const int ds = attention_decode_splits(d); ds > 0 && ds <= 65535 && !mask && workspace && !((uintptr_t)workspace & 15u) &&
+                                                   workspace_bytes >= attention_decode_workspace_bytes(d)) {
+        g.splits = ds, g.partial = (float *)workspace;
+        hipLaunchKernelGGL(attention_decode_kernel, dim3((unsigned)ds, (unsigned)stacks), dim3(AD_THREADS), 0, stream, g);
+        if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        hipLaunchKernelGGL(attention_decode_merge_kernel, dim3((unsigned)stacks), dim3(128), 0, stream, g);
+        return hipGetLastError();
+    }
     if (d.head_dim <= 64) return launch_attention_dp<64>(g, (int)stacks, stream);
     if (d.head_dim <= 96) return launch_attention_dp<96>(g, (int)stacks, stream);
     return launch_attention_dp<128>(g, (int)stacks, stream);

@@ -284,3 +284,38 @@ def test_equals_the_three_operator_sequence(device, oracle):
     three = scores.matmul(V, False, False).resolve().to(Device.CPU).storage
     fused = Q.attention(K, V, scale=1.0).resolve().to(Device.CPU).storage
     assert_close(fused, three, "fused vs three operators")
+
+
+@gpu
+def test_one_query_against_a_long_cache_streams_the_keys(device, oracle):
+    """A decode step (one query row, at least 256 cached keys, no mask tensor, a workspace) takes the streaming
+    kernel: every head dimension it serves (idle lanes past head_dim / 8), key counts off the 128-key workgroups
+    and off the 16-key loads, the cache read in place with rows past kv_len poisoned, heads merged on the way
+    out, a dominant key in the last workgroup's share, and the causal flag, which hides nothing from one query."""
+    rng = np.random.default_rng(21)
+    L = _ffi.lib()
+    for (B, H, kv_len, cap, D) in [(1, 32, 1024, 2048, 80), (2, 3, 257, 300, 8), (1, 2, 1000, 1000, 128), (1, 5, 384, 400, 64),
+                                   (1, 1, 256, 256, 96), (3, 2, 2049, 2100, 40), (1, 2, 511, 600, 72)]:
+        q = rng.standard_normal((B, H, 1, D)).astype(np.float16)
+        kc = rng.standard_normal((B, H, cap, D)).astype(np.float16)
+        vc = rng.standard_normal((B, H, cap, D)).astype(np.float16)
+        want = oracle.attention(q, kc[:, :, :kv_len], vc[:, :, :kv_len])
+        kc[:, :, kv_len:], vc[:, :, kv_len:] = np.nan, np.nan   # never read
+        Q, K, V = (Tensor.from_data(a).to(device) for a in (q, kc, vc))
+        node = Q.attention(K, V, causal=True, kv_len=kv_len)
+        need = ctypes.c_uint64()
+        assert L.rt_attention_workspace_bytes(ctypes.byref(node.op.desc), ctypes.byref(need)) == _ffi.RT_OK and need.value > 0
+        got = node.resolve().to(Device.CPU).storage
+        assert not np.isnan(got).any(), (B, H, kv_len, D)
+        assert_close(got, want, ("decode", B, H, kv_len, D))
+        single = Q.attention(K, V, kv_len=kv_len)
+        single.op.use_workspace = False                        # the tiled kernel, one pass
+        np.testing.assert_allclose(got.astype(np.float32), single.resolve().to(Device.CPU).storage.astype(np.float32),
+                                   rtol=4e-3, atol=1e-3, err_msg=str((B, H, kv_len, D)))
+        merged = Q.attention(K, V, kv_len=kv_len, merge_heads=True).resolve().to(Device.CPU).storage
+        assert np.array_equal(merged, got.transpose(0, 2, 1, 3).reshape(B, 1, H * D))
+    # a dominant key in the last share takes everything; keys that score -inf (q . k overflows to -inf) weigh nothing
+    q, k, v = rand_qkv(rng, 1, 2, 1, 700, 64)
+    q[..., 0], k[..., 0] = 30, 0
+    k[:, :, 699, 0] = 30
+    assert np.array_equal(run(device, q, k, v, scale=1.0), v[:, :, 699:700])
