@@ -414,7 +414,9 @@ RT_API rt_status rt_attention_validate(const rt_attention_desc *desc);
  * several workgroups (0 when the problem fills the device in one pass).  It pays when there are few
  * queries and many keys -- a decode step against a long cache -- where one workgroup per head would
  * leave most compute units idle.  The workspace holds partial (maximum, sum, output) triples in f32
- * between the two kernels of such a launch; its contents before and after are irrelevant. */
+ * between the two kernels of such a launch; its contents before and after are irrelevant.  With it, a
+ * launch of one query row against 256 or more keys and no mask tensor runs a streaming kernel of its
+ * own (128 keys per workgroup) instead of the tiled one. */
 RT_API rt_status rt_attention_workspace_bytes(const rt_attention_desc *desc, uint64_t *bytes);
 /* `workspace` may be NULL (or smaller than rt_attention_workspace_bytes): the launch then runs in one
  * pass.  Launches that share a workspace must not overlap. */
