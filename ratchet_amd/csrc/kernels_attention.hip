@@ -67,6 +67,27 @@ __device__ __forceinline__ int at_chunk_pos(int r, int c, int dvec) {
 // s_waitcnt vmcnt(n) lgkmcnt(0): at most n of this wavefront's loads outstanding, all LDS reads returned
 __device__ __forceinline__ constexpr int at_waitcnt(int n) { return 0x0070 | (n & 0xF) | (((n >> 4) & 0x3) << 14); }
 
+// Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the four lane groups that share a query row),
+// left in all of them: v_permlane16_swap and v_permlane32_swap of a register with itself put the partner
+// row's (half's) value beside the lane's own, so each step is two vector instructions and no trip through
+// the LDS crossbar (ds_bpermute, which __shfl_xor is, costs an LDS round trip per step).
+__device__ __forceinline__ float at_groups_max(float v) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float w = fmaxf(__builtin_bit_cast(float, (uint32_t)a[0]), __builtin_bit_cast(float, (uint32_t)a[1]));
+    const uint32_t x = __builtin_bit_cast(uint32_t, w);
+    const auto b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return fmaxf(__builtin_bit_cast(float, (uint32_t)b[0]), __builtin_bit_cast(float, (uint32_t)b[1]));
+}
+__device__ __forceinline__ float at_groups_sum(float v) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float w = __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
+    const uint32_t x = __builtin_bit_cast(uint32_t, w);
+    const auto b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
+}
+
 // DP: head_dim padded to a multiple of 32.  MASK: an additive mask tensor is present.
 // Eight wavefronts: wavefront (qt, kh) owns query tile qt (16 rows) and half kh (32 keys) of every
 // key block, with its own running maximum, sum and output; the two halves of a row are merged
@@ -240,8 +261,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
                     bmax = fmaxf(bmax, s);
                 }
         }
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, kWave));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+        bmax = at_groups_max(bmax);
         const float m_new = fmaxf(m_run, bmax);
         // a row that has seen no finite score yet keeps a reference of 0: exp2(-inf - 0) = 0
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -318,8 +338,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
             for (int r = 0; r < 4; r++) acc[d][r] = acc[d][r] * a0 + ex[(2 + 4 * d + r) * 64] * a1;
     }
     // the row's sum over its four lanes, then O / l; lane (fr, fg) holds columns 16 d + 4 fg + r of row fr
-    l_run += __shfl_xor(l_run, 16, kWave);
-    l_run += __shfl_xor(l_run, 32, kWave);
+    l_run = at_groups_sum(l_run);
     if (g.splits > 1) {
         // this workgroup saw only its share of the keys: hand (m, l, O) of every row to the merge kernel
         // (rows past q_len are never merged: a decode step has one live row of 64)
