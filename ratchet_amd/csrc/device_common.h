@@ -44,11 +44,30 @@ struct DeviceInfo {
     int num_cus = 256;
 };
 
-// Sum over the 64 lanes of a wavefront; every lane receives the total.
+// Sum / maximum over the 64 lanes of a wavefront; every lane receives the result.  Four DPP rotations
+// inside the 16-lane rows, then v_permlane16_swap and v_permlane32_swap of the register with itself (they
+// put the partner row's / half's value beside the lane's own): six vector instructions and their
+// additions, no trip through the LDS crossbar (ds_bpermute, which __shfl_xor is, costs one per step).
+template <int CTRL> __device__ __forceinline__ float wave_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <typename OP> __device__ __forceinline__ float wave_reduce(float v, OP op) {
+    v = op(v, wave_dpp<0x128>(v)); // row_ror:8
+    v = op(v, wave_dpp<0x124>(v)); // row_ror:4
+    v = op(v, wave_dpp<0x122>(v)); // row_ror:2
+    v = op(v, wave_dpp<0x121>(v)); // row_ror:1
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    v = op(__builtin_bit_cast(float, (uint32_t)a[0]), __builtin_bit_cast(float, (uint32_t)a[1]));
+    const uint32_t x = __builtin_bit_cast(uint32_t, v);
+    const auto b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return op(__builtin_bit_cast(float, (uint32_t)b[0]), __builtin_bit_cast(float, (uint32_t)b[1]));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    return wave_reduce(v, [](float a, float b) { return a + b; });
+}
+__device__ __forceinline__ float wave_max(float v) {
+    return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
 __device__ __forceinline__ float to_f32(half_t v) { return (float)v; }

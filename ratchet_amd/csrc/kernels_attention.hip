@@ -434,11 +434,6 @@ __device__ __forceinline__ float ad_row_sum(float v) {
     v += ad_dpp<0x121>(v); // row_ror:1
     return v;
 }
-__device__ __forceinline__ float ad_wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
-}
 
 __global__ __launch_bounds__(AD_THREADS) void attention_decode_kernel(AttnArgs g) {
     __shared__ float sm[4], sl[4];
@@ -483,7 +478,7 @@ __global__ __launch_bounds__(AD_THREADS) void attention_decode_kernel(AttnArgs g
         sc[i] = key0 + 16 * i < g.kv_len ? p * g.scale_log2e : -INFINITY;
         m = fmaxf(m, sc[i]);
     }
-    m = ad_wave_max(m);
+    m = wave_max(m);
     if (lane == 0) sm[wave] = m;
     __syncthreads();
     m = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));

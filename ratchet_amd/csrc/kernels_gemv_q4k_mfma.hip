@@ -143,8 +143,8 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
         float sum = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; e++) sum = __builtin_amdgcn_fdot2(half2_t{h[2 * e], h[2 * e + 1]}, one2, sum, false);
-        sum += __shfl_xor(sum, 1, kWave); // four consecutive lanes hold the four vectors of a sub-block
-        sum += __shfl_xor(sum, 2, kWave);
+        sum += wave_dpp<0xB1>(sum); // quad_perm [1,0,3,2]: four consecutive lanes hold the four vectors of a sub-block
+        sum += wave_dpp<0x4E>(sum); // quad_perm [2,3,0,1]
         if (v < nvec) {
             const int j = v >> 5, kv = v & 31;
             *(uint4_t *)(xs + j * XROW + 8 * kv) = xv[i];

@@ -18,11 +18,6 @@
 
 namespace rt {
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
-}
 
 template <typename T> struct SoftmaxVec;
 template <> struct SoftmaxVec<float> {
