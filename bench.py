@@ -741,7 +741,7 @@ def main():
             "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4),
             "traffic": GEMV_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": head["bytes"],
-            "kernel": "gemv_q8h_rowdot_kernel<5, 1, 1>",
+            "kernel": "gemv_q8h_rowdot_kernel<5, 1, 1, 4>",
         },
         "roofline_gemm": {
             "workload": gemm_f16["workload"],

@@ -44,7 +44,10 @@ struct GemvRowdotArgs {
     int has_bias, bias_on_rows, act;
 };
 
-constexpr int kRowdotWaves = 4;
+// WAVES: wavefronts per workgroup (4, 2 or 1), chosen by the launcher so that small grids still have a few workgroups
+// per compute unit: with four wavefronts the Phi-2 down-projection (2560 rows, a wavefront per row) is 640 workgroups,
+// two and a half per compute unit -- half of the chip with a third more work than the other -- and a 2560-row
+// projection at K = 2560 is 320, one and a quarter.
 
 // (q ^ 0x80) is q + 128 as an unsigned byte; 0x6400 | byte is the f16 1024 + byte; minus 1152 leaves q
 __device__ __forceinline__ void rowdot_cvt_i8x4(uint32_t v, half2_t &lo, half2_t &hi) {
@@ -71,13 +74,13 @@ template <bool WHOLE> __device__ __forceinline__ float rowdot_sum(float v) {
 // K = 512 * STEPS * SEG.  SEG == 1: a wavefront owns two rows, one per half-wave.  SEG == 2: a
 // wavefront owns one row and each half-wave half of its K.  NCT activation vectors (1 or 2).
 // Offsets inside a workgroup's rows are 32-bit; the workgroup's base is 64-bit and wave-uniform.
-template <int STEPS, int SEG, int NCT>
-__global__ __launch_bounds__(kRowdotWaves * 64) void gemv_q8h_rowdot_kernel(GemvRowdotArgs g) {
+template <int STEPS, int SEG, int NCT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int K = 512 * STEPS * SEG;
     constexpr int KQ = K / 32;
-    constexpr int THREADS = kRowdotWaves * 64;
-    constexpr int ROWS = kRowdotWaves * 2 / SEG;      // rows per workgroup
+    constexpr int THREADS = WAVES * 64;
+    constexpr int ROWS = WAVES * 2 / SEG; // rows per workgroup
     half_t *xs = (half_t *)smem;                      // [NCT][K]
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -188,36 +191,46 @@ __global__ __launch_bounds__(kRowdotWaves * 64) void gemv_q8h_rowdot_kernel(Gemv
 
 // Tunable: 1 = never take this kernel (for comparisons).
 RT_TUNABLE(g_gemv_rowdot_disable, 0);
+// Tunable: 4, 2 or 1 forces that many wavefronts per workgroup (0 = by the size of the grid).
+RT_TUNABLE(g_gemv_rowdot_waves, 0);
 
-template <int STEPS, int SEG, int NCT>
-static hipError_t launch_rowdot(dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
+template <int STEPS, int SEG, int NCT, int WAVES>
+static hipError_t launch_rowdot_w(dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
     constexpr size_t lds = (size_t)NCT * 512 * STEPS * SEG * 2;
     if constexpr (lds > 48 * 1024) {
-        const hipError_t e = ensure_lds_limit<&gemv_q8h_rowdot_kernel<STEPS, SEG, NCT>>();
+        const hipError_t e = ensure_lds_limit<&gemv_q8h_rowdot_kernel<STEPS, SEG, NCT, WAVES>>();
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((gemv_q8h_rowdot_kernel<STEPS, SEG, NCT>), grid, dim3(kRowdotWaves * 64), lds, st, g);
+    hipLaunchKernelGGL((gemv_q8h_rowdot_kernel<STEPS, SEG, NCT, WAVES>), grid, dim3(WAVES * 64), lds, st, g);
     return hipGetLastError();
 }
 
+template <int STEPS, int SEG, int NCT>
+static hipError_t launch_rowdot(int waves, dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
+    if (waves == 4) return launch_rowdot_w<STEPS, SEG, NCT, 4>(grid, st, g);
+    if (waves == 2) return launch_rowdot_w<STEPS, SEG, NCT, 2>(grid, st, g);
+    if constexpr (SEG == 1) return launch_rowdot_w<STEPS, SEG, NCT, 1>(grid, st, g);
+    return hipErrorInvalidValue;
+}
+
 template <int SEG, int NCT>
-static hipError_t launch_rowdot_steps(int steps, dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
+static hipError_t launch_rowdot_steps(int steps, int waves, dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
     if constexpr (SEG == 1) { // two half-waves per row only take over where one would need more than 10 steps
         switch (steps) {
-        case 1: return launch_rowdot<1, SEG, NCT>(grid, st, g);
-        case 2: return launch_rowdot<2, SEG, NCT>(grid, st, g);
-        case 3: return launch_rowdot<3, SEG, NCT>(grid, st, g);
-        case 4: return launch_rowdot<4, SEG, NCT>(grid, st, g);
-        case 5: return launch_rowdot<5, SEG, NCT>(grid, st, g);
+        case 1: return launch_rowdot<1, SEG, NCT>(waves, grid, st, g);
+        case 2: return launch_rowdot<2, SEG, NCT>(waves, grid, st, g);
+        case 3: return launch_rowdot<3, SEG, NCT>(waves, grid, st, g);
+        case 4: return launch_rowdot<4, SEG, NCT>(waves, grid, st, g);
+        case 5: return launch_rowdot<5, SEG, NCT>(waves, grid, st, g);
         default: break;
         }
     }
     switch (steps) {
-    case 6: return launch_rowdot<6, SEG, NCT>(grid, st, g);
-    case 7: return launch_rowdot<7, SEG, NCT>(grid, st, g);
-    case 8: return launch_rowdot<8, SEG, NCT>(grid, st, g);
-    case 9: return launch_rowdot<9, SEG, NCT>(grid, st, g);
-    case 10: return launch_rowdot<10, SEG, NCT>(grid, st, g);
+    case 6: return launch_rowdot<6, SEG, NCT>(waves, grid, st, g);
+    case 7: return launch_rowdot<7, SEG, NCT>(waves, grid, st, g);
+    case 8: return launch_rowdot<8, SEG, NCT>(waves, grid, st, g);
+    case 9: return launch_rowdot<9, SEG, NCT>(waves, grid, st, g);
+    case 10: return launch_rowdot<10, SEG, NCT>(waves, grid, st, g);
     default: return hipErrorNotSupported;
     }
 }
@@ -226,7 +239,6 @@ static hipError_t launch_rowdot_steps(int steps, dim3 grid, hipStream_t st, cons
 // hipErrorNotSupported: the shape or alignment does not fit and another kernel must run.
 hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                   hipStream_t stream, const DeviceInfo &dev) {
-    (void)dev;
     if (g_gemv_rowdot_disable) return hipErrorNotSupported;
     if (p.a_dt != RT_Q8_0H || p.act_dt != RT_F16 || p.N < 1 || p.N > 2 || p.K < 512 || p.K % 512 != 0)
         return hipErrorNotSupported;
@@ -238,7 +250,16 @@ hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B
         if (p.K % 1024 != 0 || p.K > 10240) return hipErrorNotSupported;
         seg = 2, steps = (int)(p.K / 1024);
     }
-    const int rows = kRowdotWaves * 2 / seg;
+    // wavefronts per workgroup: for one vector, the most that still give the grid three workgroups per compute unit
+    // (SEG = 2 needs a whole wavefront per row: at least two rows per workgroup there).  Measured, four / two / one:
+    // 7680 x 2560 (960 workgroups of four) 5.44 / 5.56 / 5.66 us; 2560 x 2560 (320) 3.72 / 3.81 / 3.60; 5120 x 5120
+    // (640) 7.14 / 7.00 / 7.21; 2560 x 10240 (640) 7.53 / 7.30.  With two vectors the activations a workgroup stages
+    // double and four wavefronts stay best everywhere (2560 x 10240: 9.2 against 10.9 us).
+    int waves = 4;
+    if (p.N == 1)
+        while (waves > seg && (p.M + waves * 2 / seg - 1) / (waves * 2 / seg) * p.stacks < 3 * (int64_t)dev.num_cus) waves >>= 1;
+    if (g_gemv_rowdot_waves > 0) waves = g_gemv_rowdot_waves;
+    const int rows = waves * 2 / seg;
     const int64_t groups = (p.M + rows - 1) / rows;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
 
@@ -253,8 +274,8 @@ hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B
     g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
-    if (seg == 1) return p.N == 1 ? launch_rowdot_steps<1, 1>(steps, grid, stream, g) : launch_rowdot_steps<1, 2>(steps, grid, stream, g);
-    return p.N == 1 ? launch_rowdot_steps<2, 1>(steps, grid, stream, g) : launch_rowdot_steps<2, 2>(steps, grid, stream, g);
+    if (seg == 1) return p.N == 1 ? launch_rowdot_steps<1, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<1, 2>(steps, waves, grid, stream, g);
+    return p.N == 1 ? launch_rowdot_steps<2, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<2, 2>(steps, waves, grid, stream, g);
 }
 
 } // namespace rt
