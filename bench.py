@@ -501,6 +501,17 @@ def other_configs(r: Runner, O):
     out.append(bench_generic(r, O, "C1 f32 GEMM [1500x384].[384x1536]+b", a, ffi.RT_F32, a.shape, b, b.shape, bias,
                              (False, False, False), np.float32, 1769472000, 13885440, 200, 1e-3))
     out += c3_products(r, O)
+    # the C2 shape with unquantized weights (the reference's GEMV kernels serve f32, f16 and Q8_0: ops/gemv.rs:156-574;
+    # Quantization::F16 / F32 checkpoints of Phi-2 decode through these)
+    rng = np.random.default_rng(7)
+    w = (rng.standard_normal((10240, 2560)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((1, 1, 2560)).astype(np.float32)
+    bias = rng.standard_normal(10240).astype(np.float32)
+    for name, dt, cast, tol in (("f16", ffi.RT_F16, np.float16, 2e-2), ("f32", ffi.RT_F32, np.float32, 1e-3)):
+        wb, xb, bb = w.astype(cast), x.astype(cast), bias.astype(cast)
+        out.append(bench_generic(r, O, f"C2 shape, {name} weights: x[1x2560] . W[10240x2560]^T + bias, M=1", wb, dt, wb.shape, xb,
+                                 xb.shape, bb, (False, True, True), cast, 2.0 * 10240 * 2560,
+                                 (10240 * 2560 + 2560 + 2 * 10240) * wb.itemsize, 200, tol))
     # C4's second half: the down-projection has 64 output tiles and K = 10240; with the workspace the
     # library asks for, its K is cut among four workgroups per tile (rt_matmul_enqueue_ws)
     rng = np.random.default_rng(6)
