@@ -568,8 +568,9 @@ def bench_q4k(r: Runner, O, rows, steps):
 def read_calibration(r: Runner, O, steps, warmup):
     """Context for the headline: on the same 20 rotated copies of the 27.85 MB weight and with the same graph
     timing, what a launch costs that does nothing, what one costs that only reads the buffer (consecutive
-    addresses, with and without non-temporal loads; and in the 16-row pattern the matrix-core kernel reads it
-    in), and the GEMV itself.  The probes are in ratchet_amd/libratchet_probes.so (csrc/bench_probes.hip)."""
+    addresses, with and without non-temporal loads; the same with four bytes stored per wavefront, as the GEMV
+    stores its results: a kernel that leaves modified lines in the L2s pays for their write-back when it ends; and
+    in the 16-row pattern the matrix-core kernel reads it in), and the GEMV itself.  The probes are in ratchet_amd/libratchet_probes.so (csrc/bench_probes.hip)."""
     N, K = 10240, 2560
     rng = np.random.default_rng(0)
     wbuf = O.make_q8_0h((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
@@ -580,6 +581,7 @@ def read_calibration(r: Runner, O, steps, warmup):
     vp, u64, i64 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int64
     P.probe_empty.argtypes, P.probe_read_linear.argtypes = [vp, vp], [vp, u64, ctypes.c_int, vp, vp]
     P.probe_read_rows16.argtypes = [vp, i64, i64, vp, vp]
+    P.probe_read_linear_store.argtypes = [vp, u64, vp, vp]
     stream = lambda: vp(r.torch.cuda.current_stream().cuda_stream)
     nbytes = wbuf.size - wbuf.size % 16
 
@@ -591,12 +593,14 @@ def read_calibration(r: Runner, O, steps, warmup):
     bias = rng.standard_normal(N).astype(np.float16)
     xd, bd = r.upload(x), r.upload(bias)
     out = r.torch.empty(N * 2, dtype=r.torch.uint8, device="cuda:0")
+    store_out = r.torch.empty(4 * 4 * (-(-nbytes // 5120 // 4) + 1), dtype=r.torch.uint8, device="cuda:0")  # whole workgroups of 4
     desc = r.ffi.make_desc(r.ffi.RT_Q8_0H, (N, K), r.ffi.RT_F16, (1, 1, K), False, True, True, r.ffi.RT_F16, (N,))
     rows = []
     for name, step, nb in (
             ("empty kernel (one wavefront)", lambda i: ok(P.probe_empty(vp(sink.data_ptr()), stream())), 0),
             ("read only, consecutive addresses", lambda i: ok(P.probe_read_linear(vp(ws[i].data_ptr()), nbytes, 0, vp(sink.data_ptr()), stream())), nbytes),
             ("read only, consecutive addresses, non-temporal loads", lambda i: ok(P.probe_read_linear(vp(ws[i].data_ptr()), nbytes, 1, vp(sink.data_ptr()), stream())), nbytes),
+            ("read (non-temporal) + 4 bytes stored per wavefront of 5 KiB", lambda i: ok(P.probe_read_linear_store(vp(ws[i].data_ptr()), nbytes, vp(store_out.data_ptr()), stream())), nbytes),
             ("read only, 16 rows x 64 bytes per load (the int8 codes alone)", lambda i: ok(P.probe_read_rows16(vp(ws[i].data_ptr()), N, K, vp(sink.data_ptr()), stream())), N * K),
             ("Q8_0H GEMV M=1 (the headline)", lambda i: r.enqueue(desc, ws[i], xd, bd, out), gemv_bytes(1, N, K))):
         stats = {}

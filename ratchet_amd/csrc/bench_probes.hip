@@ -14,8 +14,10 @@ __global__ void probe_empty_kernel(uint32_t *sink) {
 }
 
 // Every wavefront reads LOADS x 1 KiB of consecutive bytes, 16 per lane and load; all loads are
-// issued before the first is consumed.  NT: non-temporal loads.
-template <int LOADS, bool NT>
+// issued before the first is consumed.  NT: non-temporal loads.  STORE: one lane of every wavefront
+// also stores four bytes of what it read to out[wavefront], the way the GEMV's wavefronts store their
+// two f16 results: a kernel that leaves modified lines in the L2s pays for their write-back when it ends.
+template <int LOADS, bool NT, bool STORE>
 __global__ __launch_bounds__(256) void probe_read_linear_kernel(const probe_u4 *__restrict__ p, uint64_t nvec, uint32_t *sink) {
     const uint64_t wave = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const uint64_t base = wave * (uint64_t)(LOADS * 64) + (threadIdx.x & 63);
@@ -28,7 +30,10 @@ __global__ __launch_bounds__(256) void probe_read_linear_kernel(const probe_u4 *
     uint32_t acc = 0;
 #pragma unroll
     for (int i = 0; i < LOADS; i++) acc ^= v[i][0] ^ v[i][1] ^ v[i][2] ^ v[i][3];
-    if (acc == 0x12345678u) sink[wave & 1023] = acc; // practically never; keeps the loads alive
+    if (STORE) {
+        asm volatile("" : "+v"(acc)); // every lane's value exists here: the loads cannot move into the branch
+        if ((threadIdx.x & 63) == 0) sink[wave] = acc;
+    } else if (acc == 0x12345678u) sink[wave & 1023] = acc; // practically never; keeps the loads alive
 }
 
 // The matrix-core GEMV's address pattern: a workgroup of K / 256 wavefronts owns 16 rows of a
@@ -60,11 +65,24 @@ __attribute__((visibility("default"))) int probe_read_linear(const void *p, uint
     const unsigned blocks = (unsigned)((waves + 3) / 4);
     if (nvec == 0) return 0;
     if (nontemporal)
-        hipLaunchKernelGGL((probe_read_linear_kernel<L, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL((probe_read_linear_kernel<L, true, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
                            (const probe_u4 *)p, nvec, (uint32_t *)sink);
     else
-        hipLaunchKernelGGL((probe_read_linear_kernel<L, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL((probe_read_linear_kernel<L, false, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
                            (const probe_u4 *)p, nvec, (uint32_t *)sink);
+    return (int)hipGetLastError();
+}
+
+// reads nbytes (a multiple of 16) at p with non-temporal loads, 5 KiB per wavefront (the GEMV's share at
+// K = 2560), and stores 4 bytes per wavefront to out (at least 4 * ceil(nbytes / 5120) bytes, rounded
+// up to a multiple of 16)
+__attribute__((visibility("default"))) int probe_read_linear_store(const void *p, uint64_t nbytes, void *out, void *stream) {
+    constexpr int L = 5;
+    const uint64_t nvec = nbytes / 16, waves = (nvec + L * 64 - 1) / (L * 64);
+    const unsigned blocks = (unsigned)((waves + 3) / 4);
+    if (nvec == 0) return 0;
+    hipLaunchKernelGGL((probe_read_linear_kernel<L, true, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const probe_u4 *)p, nvec, (uint32_t *)out);
     return (int)hipGetLastError();
 }
 
