@@ -86,7 +86,11 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     const int n = lane & 15, grp = lane >> 4;
     const int64_t s = FAST ? 0 : blockIdx.y;
     const int64_t sa = g.a_stack == 1 ? 0 : s, sb = g.b_stack == 1 ? 0 : s;
-    const int64_t row0 = (int64_t)blockIdx.x * 16;
+    // workgroups go round the eight XCDs in turn: every XCD takes one run of consecutive rows, so that a line of the
+    // output is written in one XCD's L2 and leaves it whole when the kernel ends
+    const uint32_t nwg = gridDim.x;
+    const uint32_t wg = (nwg & 7) == 0 ? (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    const int64_t row0 = (int64_t)wg * 16;
     const bool live = FAST || wave < g.nsb; // padding waves (nwaves > nsb) contribute zero
     const int sbi = live ? wave : 0;
 
