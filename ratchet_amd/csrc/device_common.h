@@ -70,6 +70,21 @@ __device__ __forceinline__ float wave_max(float v) {
     return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
+// The row-streaming GEMVs' sums: the caller needs the result in one lane only, which five (six) DPP additions give.
+template <int CTRL, int ROWMASK> __device__ __forceinline__ float rowdot_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true));
+}
+// Sum over each half-wave, valid in lanes 16..31 and 48..63; with WHOLE the sum over all 64 lanes, valid in lanes 48..63.
+template <bool WHOLE> __device__ __forceinline__ float rowdot_sum(float v) {
+    v += rowdot_dpp<0x128, 0xf>(v); // row_ror:8
+    v += rowdot_dpp<0x124, 0xf>(v); // row_ror:4
+    v += rowdot_dpp<0x122, 0xf>(v); // row_ror:2
+    v += rowdot_dpp<0x121, 0xf>(v); // row_ror:1: every lane of a row of 16 holds the row's sum
+    v += rowdot_dpp<0x142, 0xa>(v); // row_bcast:15: rows 1 and 3 add the row before them
+    if (WHOLE) v += rowdot_dpp<0x143, 0xc>(v); // row_bcast:31: rows 2 and 3 add lane 31
+    return v;
+}
+
 __device__ __forceinline__ float to_f32(half_t v) { return (float)v; }
 __device__ __forceinline__ float to_f32(float v) { return v; }
 
@@ -135,6 +150,8 @@ hipError_t launch_gemv_q8h_mfma(const Problem &p, const void *A, const void *B, 
                                 hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                   hipStream_t stream, const DeviceInfo &dev);
+hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
+                                    hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                 hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,

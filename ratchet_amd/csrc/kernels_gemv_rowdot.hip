@@ -60,20 +60,6 @@ __device__ __forceinline__ void rowdot_cvt_i8x4(uint32_t v, half2_t &lo, half2_t
     hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u)) - off;
 }
 
-template <int CTRL, int ROWMASK> __device__ __forceinline__ float rowdot_dpp(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true));
-}
-// Sum over each half-wave, valid in lanes 16..31 and 48..63; with WHOLE the sum over all 64 lanes, valid in lanes 48..63.
-template <bool WHOLE> __device__ __forceinline__ float rowdot_sum(float v) {
-    v += rowdot_dpp<0x128, 0xf>(v); // row_ror:8
-    v += rowdot_dpp<0x124, 0xf>(v); // row_ror:4
-    v += rowdot_dpp<0x122, 0xf>(v); // row_ror:2
-    v += rowdot_dpp<0x121, 0xf>(v); // row_ror:1: every lane of a row of 16 holds the row's sum
-    v += rowdot_dpp<0x142, 0xa>(v); // row_bcast:15: rows 1 and 3 add the row before them
-    if (WHOLE) v += rowdot_dpp<0x143, 0xc>(v); // row_bcast:31: rows 2 and 3 add lane 31
-    return v;
-}
-
 // K = 512 * STEPS * SEG.  SEG == 1: a wavefront owns two rows, one per half-wave.  SEG == 2: a
 // wavefront owns one row and each half-wave half of its K.  NCT activation vectors (1 or 2).
 // Offsets inside a workgroup's rows are 32-bit; the workgroup's base is 64-bit and wave-uniform.

@@ -401,6 +401,46 @@ def test_float_gemv_paths(device, oracle, dt):
         assert np.array_equal(got, got2)
 
 
+@pytest.mark.parametrize("dt", [DType.F32, DType.F16], ids=["f32", "f16"])
+def test_float_row_streaming_one_vector(device, oracle, dt):
+    """f16 / f32 weights against one vector take the row-streaming kernel while a row is whole 16-byte vectors
+    and at most 10 KiB: every step count (1..10 KiB of row), rows whose last step is short or a single
+    vector, row counts off the 4 (2) rows of a workgroup, stacks of weights and of activations with
+    broadcast either way, both bias orientations and none, a fused activation; then one-hot
+    activations, which must return the weight column bit for bit."""
+    npdt = dt.numpy()
+    E = 16 // np.dtype(npdt).itemsize  # elements per 16-byte vector
+    cases = [(1, 70, 64 * E * k) for k in range(1, 11)]                       # whole steps
+    cases += [(1, 33, E), (1, 5, 63 * E), (1, 1030, 65 * E), (1, 41, 64 * E * 7 + 3 * E), (1, 1, 640 * E - E),
+              (1, 10240, 2560), (3, 19, 96 * E), (2, 9, 300 * E)]
+    for i, (S, N, K) in enumerate(cases):
+        rng = np.random.default_rng(520 + i)
+        for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
+            w = rng.standard_normal((ws, N, K)).astype(npdt)
+            x = rng.standard_normal((xs_, 1, K)).astype(npdt)
+            for to in (True, False):
+                bias = rng.standard_normal(N if to else 1).astype(npdt) if (i + to) % 3 else None
+                got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x),
+                                 None if bias is None else Tensor.from_data(bias), False, True, to)
+                want = oracle.matmul_ref(w, int(dt), w.shape, x, int(dt), x.shape, bias, False, True, to)
+                check(oracle, got, want, dt, (S, ws, xs_, N, K, to))
+    rng = np.random.default_rng(540)
+    N, K = 100, 1536
+    w, x, bias = (rng.standard_normal(sh).astype(npdt) for sh in ((N, K), (1, 1, K), (N,)))
+    for name, act in (("gelu", oracle.ACT_GELU), ("silu", oracle.ACT_SILU)):
+        y = getattr(Tensor.from_data(w).to(device).gemm(
+            Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device), False, True, True), name)().resolve()
+        want = oracle.matmul_ref(w, int(dt), w.shape, x, int(dt), x.shape, bias, False, True, True, act=act)
+        assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
+    for N, K in ((37, 2560), (6, 639 * E)):
+        w = rng.standard_normal((N, K)).astype(npdt)
+        for col in (0, K - 1, int(rng.integers(0, K))):
+            x = np.zeros((1, K), dtype=npdt)
+            x[0, col] = 1
+            got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x), None, False, True, True)
+            assert np.array_equal(got.reshape(-1), w[:, col]), (N, K, col)
+
+
 def test_empty_and_k_zero(device):
     a = Tensor.from_data(np.zeros((0, 8), np.float32))
     b = Tensor.from_data(np.zeros((8, 3), np.float32))
