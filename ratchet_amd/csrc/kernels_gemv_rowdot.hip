@@ -2,23 +2,29 @@
 //
 //   y[j, n] = sum_b d[n, b] * ( sum_{k in block b} q[n, k] * x[j, k] )  (+ bias)
 //
-// The weight matrix is read as what it is in memory, one long run of bytes: a half-wave
-// (32 lanes) owns one weight row and every load instruction fetches 512 consecutive bytes of
-// it, 16 per lane, so a wavefront touches whole 128-byte lines and touches each exactly
-// once.  That is what lets the loads be non-temporal (the stream is not kept in the
-// caches it passes through) and it is worth 0.8 us of 7.6 at the Phi-2 shape against
-// the matrix-core kernel, whose operand layout (16 rows x 64 bytes per instruction) reads
-// every line in two halves from two instructions.  Measured with that kernel's own
+// The weight matrix is read as what it is in memory, one long run of bytes: a wavefront
+// (for short rows a half-wave) owns one weight row and every load instruction fetches 1 KiB
+// (512) consecutive bytes of it, 16 per lane, so a wavefront touches whole 128-byte lines and
+// touches each exactly once.  That is what lets the loads be non-temporal (the stream is not
+// kept in the caches it passes through) and it is worth 0.8 us of 7.6 at the Phi-2 shape
+// against the matrix-core kernel, whose operand layout (16 rows x 64 bytes per instruction)
+// reads every line in two halves from two instructions.  Measured with that kernel's own
 // arithmetic on a linear address pattern: 7.56 -> 7.06 us, non-temporal 6.78 us; the
 // same non-temporal loads on the 16-row pattern: 9.05 us.
 //
 // A lane multiplies its 16 codes with the 16 activations at the same K positions:
 // the codes are widened to f16 exactly, v_dot2_f32_f16 accumulates the products in
 // f32 and the half-block's sum is scaled by the block's f16 scale in f32, so no weight is
-// rounded.  The 32 partial sums of a row meet in five DPP additions; nothing is
+// rounded.  The partial sums of a row meet in six (five) DPP additions; nothing is
 // summed across wavefronts and the kernel ends without a barrier.  The activations
 // are staged once per workgroup in LDS (their loads are issued first and the one
 // barrier waits for them only), then held in registers.
+//
+// What a launch of this kernel costs beyond reading the bytes, measured at the Phi-2
+// up-projection by taking parts away: the store of the results 0.35 us (any store: a
+// kernel that leaves modified lines in the eight L2s pays for their write-back when it
+// ends), the scales 0.45 (0.3 of it their 6 % of the bytes), staging the activations 0.2,
+// the arithmetic 0.2, the bias 0.05.
 //
 // With more vectors the dot products repeat per vector while a matrix instruction takes
 // 16 vectors at once: this kernel wins for one and two vectors (6.4 / 7.2 us against
@@ -60,16 +66,21 @@ __device__ __forceinline__ void rowdot_cvt_i8x4(uint32_t v, half2_t &lo, half2_t
     hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u)) - off;
 }
 
-// K = 512 * STEPS * SEG.  SEG == 1: a wavefront owns two rows, one per half-wave.  SEG == 2: a
-// wavefront owns one row and each half-wave half of its K.  NCT activation vectors (1 or 2).
-// Offsets inside a workgroup's rows are 32-bit; the workgroup's base is 64-bit and wave-uniform.
-template <int STEPS, int SEG, int NCT, int WAVES>
+// How a wavefront's lanes are laid over the rows and K (LAY):
+//   LAY == 1: K = 512 * STEPS; a wavefront owns two rows, one per half-wave, 512 bytes of each per step.
+//   LAY == 2: K = 1024 * STEPS; a wavefront owns one row and reads 1 KiB of it per step.
+//   LAY == 3: K = 1024 * STEPS - 512; as 2, but the last step is 512 bytes and lanes 32..63 sit it out.
+// NCT activation vectors (1 or 2).  Offsets inside a workgroup's rows are 32-bit; the workgroup's base is 64-bit
+// and wave-uniform.
+template <int STEPS, int LAY, int NCT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    constexpr int K = 512 * STEPS * SEG;
+    constexpr bool LINEAR = LAY >= 2, HALF = LAY == 3;
+    constexpr int K = LINEAR ? 1024 * STEPS - (HALF ? 512 : 0) : 512 * STEPS;
     constexpr int KQ = K / 32;
+    constexpr int KSTEP = LINEAR ? 1024 : 512;
     constexpr int THREADS = WAVES * 64;
-    constexpr int ROWS = WAVES * 2 / SEG; // rows per workgroup
+    constexpr int ROWS = LINEAR ? WAVES : WAVES * 2; // rows per workgroup
     half_t *xs = (half_t *)smem;                      // [NCT][K]
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -80,10 +91,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotA
     const uint32_t nwg = gridDim.x;
     const uint32_t wg = (nwg & 7) == 0 ? (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3) : blockIdx.x;
     const uint32_t row0 = wg * ROWS;
-    const int rw = SEG == 1 ? 2 * wave + hr : wave;                     // this lane's row within the workgroup
+    const int rw = LINEAR ? wave : 2 * wave + hr;                     // this lane's row within the workgroup
     const uint32_t last = min((uint32_t)(ROWS - 1), g.M - 1 - row0);    // rows past the end repeat the last one; never stored
     const uint32_t rc = min((uint32_t)rw, last);
-    const uint32_t kbase = SEG == 1 ? 0u : (uint32_t)hr * (512u * STEPS);
+    // this lane's offset into its row's K: k0 + KSTEP * st, but klast at the short last step of LAY 3
+    const uint32_t k0 = LINEAR ? 16u * lane : 16u * c;
+    const uint32_t klast = HALF ? 1024u * (STEPS - 1) + 16u * c : k0 + (uint32_t)(KSTEP * (STEPS - 1));
     // The bases of this workgroup's rows.  A wavefront's first load cannot leave before the scalar arithmetic in front
     // of it is done, so the terms of a stack of products (grid.y > 1) are only computed where there is one.
     const uint8_t *qbase = g.qs + (uint64_t)row0 * K;
@@ -107,17 +120,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotA
     }
     asm volatile("" ::: "memory"); // keep the loads in this order
     // 2. the weight stream: 16 bytes per lane and step, 512 consecutive bytes per half-wave
-    const uint8_t *qp = qbase + (rc * (uint32_t)K + kbase + 16u * c);
+    const uint8_t *qp = qbase + (rc * (uint32_t)K + k0);
     uint4_t w[STEPS];
 #pragma unroll
-    for (int st = 0; st < STEPS; st++) w[st] = __builtin_nontemporal_load((const uint4_t *)(qp + 512 * st));
+    for (int st = 0; st < STEPS - 1; st++) w[st] = __builtin_nontemporal_load((const uint4_t *)(qp + KSTEP * st));
+    w[STEPS - 1] = __builtin_nontemporal_load((const uint4_t *)(qbase + (rc * (uint32_t)K + klast)));
     asm volatile("" ::: "memory");
     // 3. the scale of this lane's half block at every step, then the epilogue's bias (unconditional: without
     //    a bias it reads a scale and the value is dropped; a branch here would wait for every load above)
-    const half_t *sp = sbase + (rc * (uint32_t)KQ + kbase / 32 + (c >> 1));
+    const half_t *sp = sbase + (rc * (uint32_t)KQ + (k0 >> 5));
     uint16_t dsc[STEPS];
 #pragma unroll
-    for (int st = 0; st < STEPS; st++) dsc[st] = *(const uint16_t *)(sp + 16 * st);
+    for (int st = 0; st < STEPS - 1; st++) dsc[st] = *(const uint16_t *)(sp + (KSTEP / 32) * st);
+    dsc[STEPS - 1] = *(const uint16_t *)(sbase + (rc * (uint32_t)KQ + (klast >> 5)));
     uint16_t bias_raw[NCT];
 #pragma unroll
     for (int j = 0; j < NCT; j++) {
@@ -144,14 +159,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotA
     // this lane's 16 activations per step; few enough to sit in registers while the weights are in flight
     constexpr bool HOIST = NCT * STEPS <= 6;
     uint4_t xa[HOIST ? NCT : 1][HOIST ? STEPS : 1], xb[HOIST ? NCT : 1][HOIST ? STEPS : 1];
-    const half_t *xl = xs + kbase + 16 * c;
     if (HOIST) {
 #pragma unroll
         for (int j = 0; j < NCT; j++)
 #pragma unroll
             for (int st = 0; st < STEPS; st++) {
-                xa[j][st] = *(const uint4_t *)(xl + j * K + 512 * st);
-                xb[j][st] = *(const uint4_t *)(xl + j * K + 512 * st + 8);
+                const half_t *xp = st == STEPS - 1 ? xs + klast : xs + k0 + KSTEP * st;
+                xa[j][st] = *(const uint4_t *)(xp + j * K);
+                xb[j][st] = *(const uint4_t *)(xp + j * K + 8);
             }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -167,12 +182,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotA
             const uint32_t ww = w[st][d];
             rowdot_cvt_i8x4(ww, wh[2 * d], wh[2 * d + 1]);
         }
-        const float sc = (float)__builtin_bit_cast(half_t, dsc[st]);
+        float sc = (float)__builtin_bit_cast(half_t, dsc[st]);
+        if (HALF && st == STEPS - 1 && hr) sc = 0.f; // the short last step: lanes 32..63 re-read the first half
 #pragma unroll
         for (int j = 0; j < NCT; j++) {
             uint4_t ya, yb;
             if (HOIST) ya = xa[j][st], yb = xb[j][st];
-            else ya = *(const uint4_t *)(xl + j * K + 512 * st), yb = *(const uint4_t *)(xl + j * K + 512 * st + 8);
+            else {
+                const half_t *xp = st == STEPS - 1 ? xs + klast : xs + k0 + KSTEP * st;
+                ya = *(const uint4_t *)(xp + j * K), yb = *(const uint4_t *)(xp + j * K + 8);
+            }
             float p = 0.f;
 #pragma unroll
             for (int d = 0; d < 4; d++) {
@@ -188,10 +207,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q8h_rowdot_kernel(GemvRowdotA
         }
     }
     // 6. the row's lanes meet; one lane per row writes
-    const bool writer = SEG == 1 ? c == 16 : lane == 48;
+    const bool writer = LINEAR ? lane == 48 : c == 16;
 #pragma unroll
     for (int j = 0; j < NCT; j++) {
-        const float v = rowdot_sum<SEG == 2>(acc[j]);
+        const float v = rowdot_sum<LINEAR>(acc[j]);
         if (writer && (uint32_t)rw <= last) {
             const float b = g.has_bias ? (float)__builtin_bit_cast(half_t, bias_raw[j]) : 0.f;
             op[j * ojs] = (half_t)rt_act(v + b, g.act);
@@ -204,48 +223,44 @@ RT_TUNABLE(g_gemv_rowdot_disable, 0);
 // Tunable: 4, 2 or 1 forces that many wavefronts per workgroup (0 = by the size of the grid).
 RT_TUNABLE(g_gemv_rowdot_waves, 0);
 
-template <int STEPS, int SEG, int NCT, int WAVES>
+template <int STEPS, int LAY, int NCT, int WAVES>
 static hipError_t launch_rowdot_w(dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
-    constexpr size_t lds = (size_t)NCT * 512 * STEPS * SEG * 2;
-    if constexpr (lds > 48 * 1024) {
-        const hipError_t e = ensure_lds_limit<&gemv_q8h_rowdot_kernel<STEPS, SEG, NCT, WAVES>>();
-        if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL((gemv_q8h_rowdot_kernel<STEPS, SEG, NCT, WAVES>), grid, dim3(WAVES * 64), lds, st, g);
+    constexpr size_t lds = (size_t)NCT * 2 * (LAY >= 2 ? 1024 * STEPS - (LAY == 3 ? 512 : 0) : 512 * STEPS);
+    hipLaunchKernelGGL((gemv_q8h_rowdot_kernel<STEPS, LAY, NCT, WAVES>), grid, dim3(WAVES * 64), lds, st, g);
     return hipGetLastError();
 }
 
-template <int STEPS, int SEG, int NCT>
+// The step counts each layout is built for are the ones launch_gemv_q8h_rowdot can choose.
+template <int STEPS, int LAY, int NCT>
 static hipError_t launch_rowdot(int waves, dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
-    if (waves == 4) return launch_rowdot_w<STEPS, SEG, NCT, 4>(grid, st, g);
-    if (waves == 2) return launch_rowdot_w<STEPS, SEG, NCT, 2>(grid, st, g);
-    if constexpr (SEG == 1) return launch_rowdot_w<STEPS, SEG, NCT, 1>(grid, st, g);
-    return hipErrorInvalidValue;
+    constexpr int lo = LAY == 1 ? 1 : LAY == 2 ? 4 : 5;
+    constexpr int hi = LAY == 1 ? 7 : 10;
+    if constexpr (STEPS >= lo && STEPS <= hi) {
+        if (waves == 4) return launch_rowdot_w<STEPS, LAY, NCT, 4>(grid, st, g);
+        if (waves == 2) return launch_rowdot_w<STEPS, LAY, NCT, 2>(grid, st, g);
+        if constexpr (LAY == 1) return launch_rowdot_w<STEPS, LAY, NCT, 1>(grid, st, g);
+    }
+    return hipErrorNotSupported;
 }
 
-template <int SEG, int NCT>
+template <int LAY, int NCT>
 static hipError_t launch_rowdot_steps(int steps, int waves, dim3 grid, hipStream_t st, const GemvRowdotArgs &g) {
-    if constexpr (SEG == 1) { // two half-waves per row only take over where one would need more than 10 steps
-        switch (steps) {
-        case 1: return launch_rowdot<1, SEG, NCT>(waves, grid, st, g);
-        case 2: return launch_rowdot<2, SEG, NCT>(waves, grid, st, g);
-        case 3: return launch_rowdot<3, SEG, NCT>(waves, grid, st, g);
-        case 4: return launch_rowdot<4, SEG, NCT>(waves, grid, st, g);
-        case 5: return launch_rowdot<5, SEG, NCT>(waves, grid, st, g);
-        default: break;
-        }
-    }
     switch (steps) {
-    case 6: return launch_rowdot<6, SEG, NCT>(waves, grid, st, g);
-    case 7: return launch_rowdot<7, SEG, NCT>(waves, grid, st, g);
-    case 8: return launch_rowdot<8, SEG, NCT>(waves, grid, st, g);
-    case 9: return launch_rowdot<9, SEG, NCT>(waves, grid, st, g);
-    case 10: return launch_rowdot<10, SEG, NCT>(waves, grid, st, g);
+    case 1: return launch_rowdot<1, LAY, NCT>(waves, grid, st, g);
+    case 2: return launch_rowdot<2, LAY, NCT>(waves, grid, st, g);
+    case 3: return launch_rowdot<3, LAY, NCT>(waves, grid, st, g);
+    case 4: return launch_rowdot<4, LAY, NCT>(waves, grid, st, g);
+    case 5: return launch_rowdot<5, LAY, NCT>(waves, grid, st, g);
+    case 6: return launch_rowdot<6, LAY, NCT>(waves, grid, st, g);
+    case 7: return launch_rowdot<7, LAY, NCT>(waves, grid, st, g);
+    case 8: return launch_rowdot<8, LAY, NCT>(waves, grid, st, g);
+    case 9: return launch_rowdot<9, LAY, NCT>(waves, grid, st, g);
+    case 10: return launch_rowdot<10, LAY, NCT>(waves, grid, st, g);
     default: return hipErrorNotSupported;
     }
 }
 
-// Q8_0H weights, one or two f16 activation vectors, K a multiple of 512 up to 5120 or of 1024 up to 10240.
+// Q8_0H weights, one or two f16 activation vectors, K a multiple of 512 up to 10240.
 // hipErrorNotSupported: the shape or alignment does not fit and another kernel must run.
 hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                   hipStream_t stream, const DeviceInfo &dev) {
@@ -255,21 +270,24 @@ hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B
     if (p.stacks > 65535 || p.b_ks != 1 || p.M < 1 || p.M > 0x7fffffff) return hipErrorNotSupported;
     const int64_t bjs = p.N == 1 ? 0 : p.b_js;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (bjs * 2) % 16 || (p.b_bs * 2) % 16) return hipErrorNotSupported;
-    int seg = 1, steps = (int)(p.K / 512);
-    if (steps > 10) {
-        if (p.K % 1024 != 0 || p.K > 10240) return hipErrorNotSupported;
-        seg = 2, steps = (int)(p.K / 1024);
-    }
+    if (p.K > 10240) return hipErrorNotSupported;
+    // The layout.  Short rows: a half-wave per row, so that every lane has work at every step.  From K = 4096 a
+    // wavefront per row with 1 KiB per step: half as many steps, scale loads and activation registers per lane, twice
+    // as many wavefronts.  Measured, half-wave against wavefront per row, one vector: 16384 x 512 3.5 / 4.6 us;
+    // 8192 x 1024 3.5 / 3.5; 4096 x 1536 3.2 / 3.2; 10240 x 2560 6.24 / 6.23 (and 4.9 / 5.2 with the weights in the
+    // Infinity Cache); 4096 x 4096 5.2 / 4.9; 11008 x 4096 10.0 / 9.2; 5120 x 5120 6.9 / 6.4.  Two vectors:
+    // 10240 x 2560 7.0 / 7.9; 4096 x 4096 5.9 / 5.8; 11008 x 4096 12.1 / 10.9; 5120 x 5120 8.9 / 7.5.
+    int lay = 1, steps = (int)(p.K / 512);
+    if (p.K >= 4096) lay = p.K % 1024 ? 3 : 2, steps = (int)((p.K + 512) / 1024);
+    const int rpw = lay == 1 ? 2 : 1; // rows per wavefront
     // wavefronts per workgroup: for one vector, the most that still give the grid three workgroups per compute unit
-    // (SEG = 2 needs a whole wavefront per row: at least two rows per workgroup there).  Measured, four / two / one:
-    // 7680 x 2560 (960 workgroups of four) 5.44 / 5.56 / 5.66 us; 2560 x 2560 (320) 3.72 / 3.81 / 3.60; 5120 x 5120
-    // (640) 7.14 / 7.00 / 7.21; 2560 x 10240 (640) 7.53 / 7.30.  With two vectors the activations a workgroup stages
-    // double and four wavefronts stay best everywhere (2560 x 10240: 9.2 against 10.9 us).
+    // (but at least two rows per workgroup).  With two vectors the activations a workgroup stages double and four
+    // wavefronts stay best everywhere.
     int waves = 4;
     if (p.N == 1)
-        while (waves > seg && (p.M + waves * 2 / seg - 1) / (waves * 2 / seg) * p.stacks < 3 * (int64_t)dev.num_cus) waves >>= 1;
+        while (waves * rpw > 2 && (p.M + waves * rpw - 1) / (waves * rpw) * p.stacks < 3 * (int64_t)dev.num_cus) waves >>= 1;
     if (g_gemv_rowdot_waves > 0) waves = g_gemv_rowdot_waves;
-    const int rows = waves * 2 / seg;
+    const int rows = waves * rpw;
     const int64_t groups = (p.M + rows - 1) / rows;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
 
@@ -287,8 +305,11 @@ hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B
     g.x_ss = p.b_stack == 1 ? 0 : p.b_bs, g.o_ss = p.o_bs;
     g.has_bias = p.has_bias, g.act = p.act;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
-    if (seg == 1) return p.N == 1 ? launch_rowdot_steps<1, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<1, 2>(steps, waves, grid, stream, g);
-    return p.N == 1 ? launch_rowdot_steps<2, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<2, 2>(steps, waves, grid, stream, g);
+    switch (lay) {
+    case 1: return p.N == 1 ? launch_rowdot_steps<1, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<1, 2>(steps, waves, grid, stream, g);
+    case 2: return p.N == 1 ? launch_rowdot_steps<2, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<2, 2>(steps, waves, grid, stream, g);
+    default: return p.N == 1 ? launch_rowdot_steps<3, 1>(steps, waves, grid, stream, g) : launch_rowdot_steps<3, 2>(steps, waves, grid, stream, g);
+    }
 }
 
 } // namespace rt

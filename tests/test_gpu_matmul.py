@@ -202,13 +202,14 @@ def test_q8_streaming_regular_and_ragged_variants(device, oracle):
 
 
 def test_q8_row_streaming_one_and_two_vectors(device, oracle):
-    """Q8_0H weights against one or two vectors with K a multiple of 512 take the row-streaming kernel: every
-    step count of the one-row-per-half-wave form (K = 512 .. 5120), the two-half-waves-per-row form
-    (K = 6144 .. 10240 in steps of 1024), row counts off the 8 (4) rows of a workgroup, stacks of weights and of
-    activations with broadcast either way, the bias along the rows (trans_out) and along the vectors, and a
-    fused activation; then one-hot activations, bit for bit, with -128 planted."""
+    """Q8_0H weights against one or two vectors with K a multiple of 512 up to 10240 take the row-streaming
+    kernel: every step count of the half-wave-per-row layout (K = 512 .. 3584), of the wavefront-per-row layout
+    (K = 4096 .. 10240 in steps of 1024) and of its form with a short last step (K = 4608 .. 9728), row counts off
+    the rows of a workgroup, stacks of weights and of activations with broadcast either way, the bias along the
+    rows (trans_out) and along the vectors, and a fused activation; then one-hot activations, bit for bit, with
+    -128 planted."""
     dt = DType.Q8_0H
-    cases = [(1, 1, 64, 512 * k) for k in range(1, 11)] + [(1, 1, 40, 1024 * k) for k in range(6, 11)]
+    cases = [(1, 1, 64, 512 * k) for k in range(1, 21)] + [(1, 2, 21, 512 * k) for k in (7, 8, 9, 16, 19)]
     cases += [(1, 2, 61, 2560), (1, 2, 3, 1024), (1, 1, 1, 512), (1, 2, 27, 8192), (1, 1, 10240, 2560), (1, 2, 13, 10240),
               (3, 1, 19, 1536), (2, 2, 9, 7168)]
     for i, (S, M, N, K) in enumerate(cases):
@@ -235,7 +236,7 @@ def test_q8_row_streaming_one_and_two_vectors(device, oracle):
         want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, bias, False, True, True, act=act)
         assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
     # one-hot: the dequantized weight, bit for bit, in both forms
-    for N, K in ((37, 2560), (21, 10240)):
+    for N, K in ((37, 2560), (21, 10240), (9, 4608)):
         buf = q8_weight(oracle, rng, N, K, dt)
         buf[: N * K][5::97] = 0x80
         dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
