@@ -512,6 +512,13 @@ def other_configs(r: Runner, O):
         out.append(bench_generic(r, O, f"C2 shape, {name} weights: x[1x2560] . W[10240x2560]^T + bias, M=1", wb, dt, wb.shape, xb,
                                  xb.shape, bb, (False, True, True), cast, 2.0 * 10240 * 2560,
                                  (10240 * 2560 + 2560 + 2 * 10240) * wb.itemsize, 200, tol))
+    # the Phi-2 down-projection with f16 weights: rows of 20 KiB (the looping form of the row-streaming kernel)
+    w = (rng.standard_normal((2560, 10240)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((1, 1, 10240)).astype(np.float16)
+    bias = rng.standard_normal(2560).astype(np.float16)
+    out.append(bench_generic(r, O, "down-projection shape, f16 weights: x[1x10240] . W[2560x10240]^T + bias, M=1", w, ffi.RT_F16, w.shape,
+                             x, x.shape, bias, (False, True, True), np.float16, 2.0 * 2560 * 10240,
+                             (2560 * 10240 + 10240 + 2 * 2560) * 2, 200, 2e-2))
     # C4's second half: the down-projection has 64 output tiles and K = 10240; with the workspace the
     # library asks for, its K is cut among four workgroups per tile (rt_matmul_enqueue_ws)
     rng = np.random.default_rng(6)

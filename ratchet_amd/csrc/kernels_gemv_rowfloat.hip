@@ -14,7 +14,8 @@
 // every XCD is given one run of consecutive rows and an output line leaves one L2 whole.
 //
 // Measured at 10240 x 2560: f16 13.1 -> 9.1 us (0.72 of the HBM peak), f32 23.1 -> 16.6 us (0.79) against the one-load-at-a-time
-// kernel in kernels_gemv.hip, which keeps every other shape (more vectors, longer or unaligned rows).
+// kernel in kernels_gemv.hip, which keeps every other shape (more vectors, unaligned rows).  Rows longer than
+// 10 KiB (up to 64) take the looping form of the same stream, gemv_float_rowlong_kernel.
 //
 // Roles in the reference: ops/gemv.rs:156-331 (workgroup GEMV), ops/gemv.rs:333-558 (subgroup GEMV).
 #include "device_common.h"
@@ -116,8 +117,98 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_float_rowdot_kernel(GemvRowFl
     }
 }
 
-// Tunable: 1 = never take this kernel (for comparisons).
+
+// Rows longer than 10 KiB: the same wavefront-per-row stream in passes of 8 KiB, the next pass's loads in flight while
+// this one is multiplied (two register sets).  Loads past the end of the row re-read its last vector and their
+// products are dropped, so the loop has no branch around a load.  The activations stay in LDS (up to 64 KiB).
+constexpr int kRowLongSteps = 8;
+
+template <typename AT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_float_rowlong_kernel(GemvRowFloatArgs g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int THREADS = WAVES * 64, PS = kRowLongSteps;
+    uint4_t *xs = (uint4_t *)smem; // [nvec]
+    const int t = threadIdx.x, lane = t & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t nwg = gridDim.x;
+    const uint32_t wg = (nwg & 7) == 0 ? (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    const uint32_t row0 = wg * WAVES;
+    const uint32_t last = min((uint32_t)(WAVES - 1), g.M - 1 - row0);
+    const uint32_t rc = min(wave, last);
+    const uint8_t *abase = g.A + (uint64_t)(row0 + rc) * g.a_rs;
+    const uint8_t *xg = g.X;
+    AT *obase = (AT *)g.out;
+    if (blockIdx.y != 0) {
+        asm volatile("" ::: "memory");
+        const int64_t s = blockIdx.y;
+        abase += s * g.a_ss, xg += s * g.x_ss, obase += s * g.o_ss;
+    }
+    const uint32_t nvec = g.nvec;
+    const uint32_t npass = (nvec + 64 * PS - 1) / (64 * PS);
+
+    uint4_t w0[PS], w1[PS];
+    auto issue = [&](uint4_t (&w)[PS], uint32_t pass) __attribute__((always_inline)) {
+#pragma unroll
+        for (int st = 0; st < PS; st++) {
+            const uint32_t i = min(64u * (pass * PS + st) + lane, nvec - 1);
+            w[st] = __builtin_nontemporal_load((const uint4_t *)(abase + 16 * (size_t)i));
+        }
+    };
+    // the activations first (they come from the L2), then the first pass of the row
+    for (uint32_t v0 = 0; v0 < nvec; v0 += 4 * THREADS) {
+        uint4_t xv[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) xv[i] = *(const uint4_t *)(xg + 16 * (size_t)min(v0 + i * THREADS + t, nvec - 1));
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (v0 + i * THREADS + t < nvec) xs[v0 + i * THREADS + t] = xv[i];
+    }
+    issue(w0, 0);
+    const AT braw = *(const AT *)(g.bias + sizeof(AT) * (size_t)((row0 + rc) * g.bias_rs));
+    AT *op = obase + (int64_t)(row0 + wave) * g.o_is;
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the barrier waits for the LDS writes, not for the row
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+
+    float acc = 0.f;
+    auto multiply = [&](const uint4_t (&w)[PS], uint32_t pass) __attribute__((always_inline)) {
+#pragma unroll
+        for (int st = 0; st < PS; st++) {
+            const uint32_t i = 64u * (pass * PS + st) + lane;
+            const uint4_t xv = xs[min(i, nvec - 1)];
+            float p = 0.f;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t ww = w[st][d], xw = xv[d];
+                if constexpr (sizeof(AT) == 2) p = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ww), __builtin_bit_cast(half2_t, xw), p, false);
+                else p = fmaf(__builtin_bit_cast(float, ww), __builtin_bit_cast(float, xw), p);
+            }
+            acc += i < nvec ? p : 0.f;
+        }
+    };
+    for (uint32_t pass = 0; pass < npass; pass += 2) {
+        issue(w1, pass + 1); // past the last pass: re-reads the row's end, dropped
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(w0, pass);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(w0, pass + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(w1, pass + 1); // contributes nothing past the last pass
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const float v = rowdot_sum<true>(acc);
+    if (lane == 63 && wave <= last) {
+        const float b = g.has_bias ? to_f32(braw) : 0.f;
+        *op = from_f32<AT>(rt_act(v + b, g.act));
+    }
+}
+
+// Tunable: 1 = never take these kernels (for comparisons).
 RT_TUNABLE(g_gemv_rowfloat_disable, 0);
+// Tunable: wavefronts (= rows) per workgroup, 0 = by the size of the grid.
+RT_TUNABLE(g_gemv_rowfloat_waves, 0);
 
 template <typename AT, int STEPS, int WAVES>
 static hipError_t launch_rowfloat_w(dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
@@ -128,6 +219,11 @@ static hipError_t launch_rowfloat_w(dim3 grid, size_t lds, hipStream_t st, const
 template <typename AT, int STEPS>
 static hipError_t launch_rowfloat(int waves, dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
     if (waves == 4) return launch_rowfloat_w<AT, STEPS, 4>(grid, lds, st, g);
+#ifdef RT_DEV_TUNABLES
+    if (waves == 8) return launch_rowfloat_w<AT, STEPS, 8>(grid, lds, st, g);
+    if (waves == 5) return launch_rowfloat_w<AT, STEPS, 5>(grid, lds, st, g);
+    if (waves == 10) return launch_rowfloat_w<AT, STEPS, 10>(grid, lds, st, g);
+#endif
     return launch_rowfloat_w<AT, STEPS, 2>(grid, lds, st, g);
 }
 
@@ -148,7 +244,27 @@ static hipError_t launch_rowfloat_steps(int steps, int waves, dim3 grid, size_t 
     }
 }
 
-// f16 or f32 weights with rows of whole 16-byte vectors, at most 10 KiB long, one activation vector of the same type.
+template <typename AT, int WAVES>
+static hipError_t launch_rowlong_w(dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
+    if (lds > 48 * 1024) {
+        const hipError_t e = ensure_lds_limit<&gemv_float_rowlong_kernel<AT, WAVES>>();
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((gemv_float_rowlong_kernel<AT, WAVES>), grid, dim3(WAVES * 64), lds, st, g);
+    return hipGetLastError();
+}
+
+static hipError_t launch_rowlong(bool f16, int waves, dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
+#ifdef RT_DEV_TUNABLES
+    if (f16 && waves == 8) return launch_rowlong_w<half_t, 8>(grid, lds, st, g);
+    if (f16 && waves == 5) return launch_rowlong_w<half_t, 5>(grid, lds, st, g);
+    if (f16 && waves == 10) return launch_rowlong_w<half_t, 10>(grid, lds, st, g);
+#endif
+    if (f16) return waves == 4 ? launch_rowlong_w<half_t, 4>(grid, lds, st, g) : launch_rowlong_w<half_t, 2>(grid, lds, st, g);
+    return waves == 4 ? launch_rowlong_w<float, 4>(grid, lds, st, g) : launch_rowlong_w<float, 2>(grid, lds, st, g);
+}
+
+// f16 or f32 weights with rows of whole 16-byte vectors, at most 64 KiB long, one activation vector of the same type.
 // hipErrorNotSupported: the shape or alignment does not fit and another kernel must run.
 hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                     hipStream_t stream, const DeviceInfo &dev) {
@@ -157,7 +273,7 @@ hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void 
     if (p.stacks > 65535 || p.a_ks != 1 || p.b_ks != 1 || p.M < 1 || p.M > 0x7fffffff) return hipErrorNotSupported;
     const int64_t esz = p.act_dt == RT_F16 ? 2 : 4;
     const int64_t row_bytes = p.K * esz;
-    if (row_bytes < 16 || row_bytes % 16 != 0 || row_bytes > 10 * 1024) return hipErrorNotSupported;
+    if (row_bytes < 16 || row_bytes % 16 != 0 || row_bytes > 64 * 1024) return hipErrorNotSupported;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (p.a_rs * esz) % 16 || (p.a_bs * esz) % 16 || (p.b_bs * esz) % 16)
         return hipErrorNotSupported;
     const uint32_t nvec = (uint32_t)(row_bytes / 16);
@@ -165,6 +281,7 @@ hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void 
     // four rows per workgroup; two where that leaves the grid under three workgroups per compute unit
     int waves = 4;
     if ((p.M + 3) / 4 * p.stacks < 3 * (int64_t)dev.num_cus) waves = 2;
+    if (g_gemv_rowfloat_waves > 0) waves = g_gemv_rowfloat_waves;
     const int64_t groups = (p.M + waves - 1) / waves;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
 
@@ -179,6 +296,7 @@ hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void 
     g.has_bias = p.has_bias, g.act = p.act;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
     const size_t lds = (size_t)nvec * 16;
+    if (steps > 10) return launch_rowlong(p.act_dt == RT_F16, waves, grid, lds, stream, g);
     return p.act_dt == RT_F16 ? launch_rowfloat_steps<half_t>(steps, waves, grid, lds, stream, g)
                               : launch_rowfloat_steps<float>(steps, waves, grid, lds, stream, g);
 }

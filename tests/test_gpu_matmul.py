@@ -404,9 +404,9 @@ def test_float_gemv_paths(device, oracle, dt):
 
 @pytest.mark.parametrize("dt", [DType.F32, DType.F16], ids=["f32", "f16"])
 def test_float_row_streaming_one_vector(device, oracle, dt):
-    """f16 / f32 weights against one vector take the row-streaming kernel while a row is whole 16-byte vectors
-    and at most 10 KiB: every step count (1..10 KiB of row), rows whose last step is short or a single
-    vector, row counts off the 4 (2) rows of a workgroup, stacks of weights and of activations with
+    """f16 / f32 weights against one vector take the row-streaming kernels while a row is whole 16-byte vectors
+    and at most 64 KiB: every step count (1..10 KiB of row), rows whose last step is short or a single
+    vector, longer rows (the form that loops over 8 KiB passes), row counts off the 4 (2) rows of a workgroup, stacks of weights and of activations with
     broadcast either way, both bias orientations and none, a fused activation; then one-hot
     activations, which must return the weight column bit for bit."""
     npdt = dt.numpy()
@@ -414,6 +414,8 @@ def test_float_row_streaming_one_vector(device, oracle, dt):
     cases = [(1, 70, 64 * E * k) for k in range(1, 11)]                       # whole steps
     cases += [(1, 33, E), (1, 5, 63 * E), (1, 1030, 65 * E), (1, 41, 64 * E * 7 + 3 * E), (1, 1, 640 * E - E),
               (1, 10240, 2560), (3, 19, 96 * E), (2, 9, 300 * E)]
+    # rows longer than 10 KiB (the looping form): one vector past it, an odd and an even number of 8 KiB passes, 64 KiB
+    cases += [(1, 37, 641 * E), (1, 300, 1024 * E), (1, 6, 1537 * E), (1, 5, 4096 * E), (2, 7, 700 * E), (1, 2560, 10240)]
     for i, (S, N, K) in enumerate(cases):
         rng = np.random.default_rng(520 + i)
         for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
@@ -423,7 +425,15 @@ def test_float_row_streaming_one_vector(device, oracle, dt):
                 bias = rng.standard_normal(N if to else 1).astype(npdt) if (i + to) % 3 else None
                 got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x),
                                  None if bias is None else Tensor.from_data(bias), False, True, to)
-                want = oracle.matmul_ref(w, int(dt), w.shape, x, int(dt), x.shape, bias, False, True, to)
+                if dt == DType.F32 and K >= 8192:
+                    # the oracle sums K products one after the other in f32: at this K its own rounding reaches the
+                    # tolerance on outputs near zero, so the exact (f64) product is the reference here
+                    want = np.einsum("snk,sk->sn", np.broadcast_to(w, (S, N, K)).astype(np.float64),
+                                     np.broadcast_to(x[:, 0], (S, K)).astype(np.float64))
+                    want = want + (0 if bias is None else bias.astype(np.float64))
+                    want = want[:, None, :] if to else want[:, :, None]
+                else:
+                    want = oracle.matmul_ref(w, int(dt), w.shape, x, int(dt), x.shape, bias, False, True, to)
                 check(oracle, got, want, dt, (S, ws, xs_, N, K, to))
     rng = np.random.default_rng(540)
     N, K = 100, 1536
