@@ -569,6 +569,11 @@ def bench_q4k(r: Runner, O, rows, steps):
         out.append(bench_generic(r, O, f"C5 Q4_K M={M} x[{M}x3072].W[8192x3072]^T", blocks, ffi.RT_Q4_K, (8192, 3072), x,
                                  x.shape, None, (False, True, True), np.float16, 50331648 * M,
                                  14155776 + 6144 * M + 16384 * M, steps, 2e-2))
+    # a down-projection with K = 8192 (Phi-3-mini's, phi3/mlp.rs): rows of 32 super-blocks, one vector
+    blocks = O.q4k_quantize((rng.standard_normal((3072, 8192)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((1, 1, 8192)).astype(np.float16)
+    out.append(bench_generic(r, O, "Q4_K M=1, K = 8192: x[1x8192].W[3072x8192]^T", blocks, ffi.RT_Q4_K, (3072, 8192), x, x.shape,
+                             None, (False, True, True), np.float16, 2.0 * 3072 * 8192, 3072 * 32 * 144 + 2 * 8192 + 2 * 3072, steps, 2e-2))
     return out
 
 

@@ -152,6 +152,8 @@ hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B
                                   hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                     hipStream_t stream, const DeviceInfo &dev);
+hipError_t launch_gemv_q4k_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
+                                  hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                 hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,

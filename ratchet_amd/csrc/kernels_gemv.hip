@@ -318,7 +318,10 @@ hipError_t launch_gemv(const Problem &p, const void *A, const void *B, const voi
         if (e != hipErrorNotSupported) return e;
     }
     if (p.kernel == RT_KERNEL_GEMV_Q4K) {
-        hipError_t e = launch_gemv_q4k_mfma(p, A, B, bias, out, stream, dev);
+        // one vector: the row-streaming kernel; then the matrix-core kernel
+        hipError_t e = launch_gemv_q4k_rowdot(p, A, B, bias, out, stream, dev);
+        if (e != hipErrorNotSupported) return e;
+        e = launch_gemv_q4k_mfma(p, A, B, bias, out, stream, dev);
         if (e != hipErrorNotSupported) return e;
     }
     if (p.kernel == RT_KERNEL_GEMV_FLOAT) { // one vector, rows of whole 16-byte vectors up to 10 KiB: the row-streaming kernel

@@ -352,6 +352,46 @@ def test_q4k_streaming_shapes(device, oracle):
     check(oracle, got, want, DType.F16, "no trans_out")
 
 
+def test_q4k_row_streaming_long_rows(device, oracle):
+    """Q4_K weights with K above 4096 against one vector take the row-streaming kernel (a wavefront per row, the
+    row read as a run of 16-byte vectors, block headers handed to the lanes of their blocks through LDS): K from
+    4352 to 10752 (three to six steps of 64 vectors, the last one short or whole), row counts off the 16 / 8 / 4
+    rows of a workgroup, both bias orientations and none, stacks of weights and of activations with broadcast
+    either way, a fused activation; then one-hot activations, which must return the dequantized column bit for bit."""
+    cases = [(1, 50, 4352), (1, 9, 5120), (1, 1, 6144), (1, 37, 8192), (1, 130, 10752), (1, 3072, 8192), (3, 7, 4608),
+             (2, 21, 7168)]
+    for i, (S, N, K) in enumerate(cases):
+        rng = np.random.default_rng(470 + i)
+        for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
+            blocks = oracle.q4k_quantize((rng.standard_normal((ws, N, K)) * 0.02).astype(np.float32))
+            x = rng.standard_normal((xs_, 1, K)).astype(np.float16)
+            for to in (True, False):
+                bias = rng.standard_normal(N if to else 1).astype(np.float16) if (i + to) % 3 else None
+                got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (ws, N, K)), Tensor.from_data(x),
+                                 None if bias is None else Tensor.from_data(bias), False, True, to)
+                want = oracle.matmul_ref(blocks, oracle.Q4_K, (ws, N, K), x, oracle.F16, x.shape, bias, False, True, to)
+                check(oracle, got, want, DType.F16, (S, ws, xs_, N, K, to))
+    rng = np.random.default_rng(480)
+    N, K = 100, 4864
+    blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((1, 1, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    for name, act in (("gelu", oracle.ACT_GELU), ("silu", oracle.ACT_SILU)):
+        y = getattr(Tensor.from_quantized(blocks, DType.Q4_K, (N, K)).to(device).gemm(
+            Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device), False, True, True), name)().resolve()
+        want = oracle.matmul_ref(blocks, oracle.Q4_K, (N, K), x, oracle.F16, x.shape, bias, False, True, True, act=act)
+        assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
+    for N, K in ((23, 8192), (5, 4352)):
+        blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+        dq = oracle.q4k_dequantize(blocks).reshape(N, K)
+        for col in (0, K - 1, 255, 256, 4096 + 31, int(rng.integers(0, K)), int(rng.integers(0, K))):
+            x = np.zeros((1, K), dtype=np.float16)
+            x[0, col] = 1
+            got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (N, K)), Tensor.from_data(x), None,
+                             False, True, True)
+            assert np.array_equal(got.reshape(-1), dq[:, col].astype(np.float16)), (N, K, col)
+
+
 def test_q4k_one_hot_is_bit_exact_dequant(device, oracle):
     rng = np.random.default_rng(401)
     N, K = 40, 512
