@@ -518,28 +518,32 @@ __global__ __launch_bounds__(AD_THREADS) void attention_decode_kernel(AttnArgs g
 __global__ __launch_bounds__(128) void attention_decode_merge_kernel(AttnArgs g) {
     const int bh = blockIdx.x, b = bh / g.heads, h = bh - b * g.heads, d = threadIdx.x;
     const float *base = g.partial + (size_t)bh * g.splits * AD_PSTRIDE;
-    // running (maximum, sum, output), sixteen splits' values requested at a time: the partial results come
-    // from other XCDs' workgroups, so every round of loads is a trip to memory, and a cache of 2048 keys is one round
+    // (maximum, sum, output) over the splits, sixteen splits' values requested at a time: the partial results come
+    // from other XCDs' workgroups, so every round of loads is a trip to memory, and a cache of 2048 keys is one round.
+    // Within a round the sixteen weights are independent of each other (one maximum first, then sixteen
+    // exponentials side by side), not a chain of sixteen rescalings.
     float m = -INFINITY, l = 0.f, o = 0.f;
     const int dc = min(d, g.D - 1);
     for (int s0 = 0; s0 < g.splits; s0 += 16) {
         float ms[16], ls[16], os[16];
 #pragma unroll
         for (int u = 0; u < 16; u++) {
-            const float *ps = base + (size_t)min(s0 + u, g.splits - 1) * AD_PSTRIDE; // past the last split: re-read it, skipped below
-            ms[u] = ps[0], ls[u] = ps[1], os[u] = ps[4 + dc];
+            const float *ps = base + (size_t)min(s0 + u, g.splits - 1) * AD_PSTRIDE; // past the last split: re-read it, weight 0 below
+            ms[u] = s0 + u < g.splits ? ps[0] : -INFINITY, ls[u] = ps[1], os[u] = ps[4 + dc];
         }
+        float m_new = m;
+#pragma unroll
+        for (int u = 0; u < 16; u++) m_new = fmaxf(m_new, ms[u]);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float a = __builtin_amdgcn_exp2f(m - m_use);
+        float lr = 0.f, orr = 0.f;
 #pragma unroll
         for (int u = 0; u < 16; u++) {
-            if (s0 + u < g.splits) {
-                const float m_new = fmaxf(m, ms[u]);
-                const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                const float a = __builtin_amdgcn_exp2f(m - m_use), w = __builtin_amdgcn_exp2f(ms[u] - m_use);
-                l = l * a + ls[u] * w;
-                o = o * a + os[u] * w;
-                m = m_new;
-            }
+            const float w = __builtin_amdgcn_exp2f(ms[u] - m_use); // exp2(-inf) = 0: a split past the end, or one with no visible key
+            lr = fmaf(ls[u], w, lr), orr = fmaf(os[u], w, orr);
         }
+        l = fmaf(l, a, lr), o = fmaf(o, a, orr);
+        m = m_new;
     }
     if (d < g.D) g.O[b * g.o_bs + h * g.o_hs + d] = (half_t)(o / l); // no visible key anywhere: 0 / 0 = NaN, as in the single pass
 }
