@@ -42,6 +42,7 @@ struct GemvMfmaArgs {
     int64_t M, K;          // weight rows, contraction (K % 256 == 0)
     int NC;                // activation vectors (1..16)
     int nunits;            // K / 256
+    int rows_wg;           // weight rows per workgroup: at most 16 * RG, a multiple of 8
     int64_t a_stack, b_stack;
     int64_t b_bs, b_js;
     int64_t o_bs, o_is, o_js;
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
     const int64_t s = FAST ? 0 : blockIdx.y;
     // an operand's stack is either the full stack or 1 (broadcast)
     const int64_t sa = g.a_stack == 1 ? 0 : s, sb = g.b_stack == 1 ? 0 : s;
-    const int64_t row0 = (int64_t)blockIdx.x * (16 * RG);
+    const int64_t row0 = (int64_t)blockIdx.x * (FAST ? 16 * RG : g.rows_wg);
     const int u0 = wave * UPW;                            // first unit of this wave
     const int nu = FAST ? UPW : min(UPW, g.nunits - u0);  // units this wave really has (<= 0 for a padding wave)
     const int u0c = nu > 0 ? u0 : 0;                      // a padding wave reads unit 0 and discards the result
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
         // (a wave-uniform 64-bit base plus a 32-bit lane offset: K <= 16384, so 64 rows stay below 2^20)
         const uint8_t *qbase = g.qs + (sa * g.M + row0) * g.K + (int64_t)u0c * kUnitK;
         const half_t *sbase = g.scales + (sa * g.M + row0) * (int64_t)kq + (int64_t)u0c * 8;
-        const int last = (int)min((int64_t)(16 * RG - 1), g.M - 1 - row0); // rows past the end duplicate the last one; never stored
+        const int last = (int)min((int64_t)(g.rows_wg - 1), g.M - 1 - row0); // rows past the workgroup's or the matrix's end duplicate the last one; never stored
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             const uint32_t rowl = (uint32_t)min(16 * rg + n, last);
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
         // compiler wait for every outstanding load right after issuing this one.
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
-            const int64_t bi = g.bias_on_rows ? min(row0 + 16 * rg + (t & 15), g.M - 1) : (int64_t)min((t >> 4) & 15, g.NC - 1);
+            const int64_t bi = g.bias_on_rows ? min(row0 + min(16 * rg + (t & 15), g.rows_wg - 1), g.M - 1) : (int64_t)min((t >> 4) & 15, g.NC - 1);
             const half_t *bp = g.has_bias ? g.bias + bi : sbase;
             bias_raw[rg] = *(const uint16_t *)bp;
         }
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
             float v = 0.f;
             for (int w2 = 0; w2 < nwaves; w2++) v += psum[(w2 * RG + rg) * 256 + t];
             const int64_t i = row0 + 16 * rg + (t & 15);
-            if (FAST || (j < g.NC && i < g.M)) g.out[s * g.o_bs + i * g.o_is + j * g.o_js] = (half_t)rt_act(v + (g.has_bias ? (float)__builtin_bit_cast(half2_t, bias_raw[rg])[0] : 0.f), g.act);
+            if (FAST || (j < g.NC && i < g.M && 16 * rg + (t & 15) < g.rows_wg)) g.out[s * g.o_bs + i * g.o_is + j * g.o_js] = (half_t)rt_act(v + (g.has_bias ? (float)__builtin_bit_cast(half2_t, bias_raw[rg])[0] : 0.f), g.act);
         }
     }
 }
@@ -310,6 +311,9 @@ static hipError_t launch_rg(int rg, dim3 grid, int nwaves, size_t lds, hipStream
     switch (rg) {
     case 1: return launch_nc<UPW, 1>(grid, nwaves, lds, st, g);
     case 2: return launch_nc<UPW, 2>(grid, nwaves, lds, st, g);
+    case 3:
+        if constexpr (UPW == 1) return launch_nc<UPW, 3>(grid, nwaves, lds, st, g);
+        return hipErrorInvalidValue;
     case 4: return launch_nc<UPW, 4>(grid, nwaves, lds, st, g);
     default: return hipErrorInvalidValue;
     }
@@ -346,15 +350,32 @@ hipError_t launch_gemv_q8h_mfma(const Problem &p, const void *A, const void *B, 
     int nwaves = (g.nunits + upw - 1) / upw;
     if (nwaves > 16) return hipErrorNotSupported; // K > 16384
     if (nwaves < 4) nwaves = 4;                   // the final sum uses 256 threads
-    // Row groups per workgroup: one measured best at every vector count (more groups per
-    // workgroup mean more loads per wavefront and a longer tail after the last one returns).
-    int rg = g_gemv_mfma_rg;
-    if (rg == 0) rg = 1;
-    (void)dev;
+    // Rows per workgroup.  16 (one MFMA row group) while all workgroups are resident at once: more groups per
+    // workgroup mean more loads per wavefront and a longer tail after the last one returns.  With many vectors the
+    // activations' LDS leaves room for two workgroups per compute unit, or one, and the grid then runs in rounds
+    // (10240 rows, 16 vectors: 640 workgroups, one per compute unit = 3 rounds, 13.2 us).  There every compute unit
+    // gets one workgroup with its share of the rows, ceil(rows / num_cus) rounded up to 8, in up to four row groups
+    // the last of which may be half empty (40 rows per workgroup: 10.5 us; 9 / 12 vectors 11.0 / 11.4 -> 10.3 / 10.4;
+    // two workgroups of 24 rows per compute unit measured slower than either, 12.3 us at 9 vectors).
+    int rg = g_gemv_mfma_rg, rows_wg = 0;
+    if (rg == 0) {
+        rg = 1;
+        const size_t lds_x = (size_t)nwaves * g.NC * (upw * kUnitK + kXPad) * 2;
+        auto fit = [&](int r) { // workgroups of r row groups that fit a compute unit
+            const int by_lds = (int)((160 * 1024) / (lds_x + (size_t)nwaves * r * 1024)), by_waves = 32 / nwaves;
+            return by_lds < by_waves ? by_lds : by_waves;
+        };
+        if (upw == 1 && p.stacks == 1 && (p.M + 15) / 16 > (int64_t)dev.num_cus * fit(1)) {
+            const int64_t per = ((p.M + dev.num_cus - 1) / dev.num_cus + 7) & ~(int64_t)7;
+            if (per <= 64 && fit((int)(per + 15) / 16) >= 1) rows_wg = (int)per, rg = (rows_wg + 15) / 16;
+        }
+    }
     if (upw * rg > 4) rg = 4 / upw > 0 ? 4 / upw : 1; // at most 16 weight loads in flight per lane
+    if (rows_wg == 0 || rows_wg > 16 * rg) rows_wg = 16 * rg;
+    g.rows_wg = rows_wg;
     const size_t lds = (size_t)nwaves * g.NC * (upw * kUnitK + kXPad) * 2 + (size_t)nwaves * rg * 1024;
     if (lds > 160 * 1024) return hipErrorNotSupported;
-    const int64_t groups = (p.M + 16 * rg - 1) / (16 * rg);
+    const int64_t groups = (p.M + rows_wg - 1) / rows_wg;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
     switch (upw) {

@@ -201,6 +201,32 @@ def test_q8_streaming_regular_and_ragged_variants(device, oracle):
     assert np.array_equal(got, dq[:, cols].T.astype(adt))
 
 
+def test_q8_streaming_rows_dealt_one_workgroup_per_compute_unit(device, oracle):
+    """With 9..16 vectors the activations' LDS lets one or two workgroups of the Q8_0H streaming kernel live on a
+    compute unit; when the 16-row workgroups would then run in rounds, every compute unit gets one workgroup with
+    its share of the rows instead (24, 40 or 48 of them: row groups whose last one is half empty or ragged)."""
+    dt = DType.Q8_0H
+    for i, (M, N, K) in enumerate([(16, 4104, 2560), (9, 10240, 2560), (13, 10248, 2560)]):
+        rng = np.random.default_rng(290 + i)
+        buf = q8_weight(oracle, rng, N, K, dt)
+        x = rng.standard_normal((1, M, K)).astype(np.float16)
+        for to in (True, False):
+            bias = rng.standard_normal(N if to else M).astype(np.float16)
+            got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (N, K)), Tensor.from_data(x), Tensor.from_data(bias),
+                             False, True, to)
+            want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, bias, False, True, to)
+            check(oracle, got, want, DType.F16, (M, N, K, to))
+    # one-hot activations: every row of the weight, bit for bit, through the half-empty row group
+    N, K = 4104, 2560
+    buf = q8_weight(oracle, np.random.default_rng(295), N, K, dt)
+    dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
+    cols = np.arange(16) * 157 + 3
+    x = np.zeros((16, K), dtype=np.float16)
+    x[np.arange(16), cols] = 1
+    got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (N, K)), Tensor.from_data(x), None, False, True, True)
+    assert np.array_equal(got, dq[:, cols].T.astype(np.float16))
+
+
 def test_q8_row_streaming_one_and_two_vectors(device, oracle):
     """Q8_0H weights against one or two vectors with K a multiple of 512 up to 10240 take the row-streaming
     kernel: every step count of the half-wave-per-row layout (K = 512 .. 3584), of the wavefront-per-row layout
