@@ -32,6 +32,7 @@ struct GemvQ4kArgs {
     int64_t M, K;
     int NC;     // activation vectors (1..16)
     int nsb;    // super-blocks per row
+    int rows_wg; // weight rows per workgroup: at most 16 * RG, a multiple of 8
     int64_t a_stack, b_stack;
     int64_t b_bs, b_js;
     int64_t o_bs, o_is, o_js;
@@ -72,7 +73,9 @@ __device__ __forceinline__ half8_t q4k_scaled(uint32_t v0, uint32_t v1, half_t s
 // wavefront per super-block column, exactly NCT vectors, all offsets below 2^31.  Its prologue
 // is a handful of 32-bit operations; the kernel is bound by instruction issue (several
 // wavefronts per SIMD run the same instructions at the same time), so that shows.
-template <int NCT, bool FAST>
+// RG: 16-row groups per workgroup (1 or 2).  They share the staged activations; with 9..16 vectors those leave room
+// for one workgroup per compute unit, and two row groups then cover 8192 rows in one round of 256 workgroups.
+template <int NCT, bool FAST, int RG>
 __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int XROW = 256 + kQ4kXPad; // halfs per staged activation row (one super-block of K)
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     const int NC = FAST ? NCT : g.NC;
     half_t *xs = (half_t *)smem + (size_t)wave * NC * (XROW + 16); // [NC][XROW] then [NC][2][8] sub-block sums
     half_t *sxs = xs + (size_t)NC * XROW;
-    float *psum = (float *)((half_t *)smem + (size_t)nwaves * NC * (XROW + 16)); // [nwaves][256]
+    float *psum = (float *)((half_t *)smem + (size_t)nwaves * NC * (XROW + 16)); // [nwaves][RG][256]
 
     const int n = lane & 15, grp = lane >> 4;
     const int64_t s = FAST ? 0 : blockIdx.y;
@@ -90,15 +93,15 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     // output is written in one XCD's L2 and leaves it whole when the kernel ends
     const uint32_t nwg = gridDim.x;
     const uint32_t wg = (nwg & 7) == 0 ? (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3) : blockIdx.x;
-    const int64_t row0 = (int64_t)wg * 16;
+    const int64_t row0 = (int64_t)wg * (FAST ? 16 * RG : g.rows_wg);
     const bool live = FAST || wave < g.nsb; // padding waves (nwaves > nsb) contribute zero
     const int sbi = live ? wave : 0;
 
     // 1. this wave's 256 activations per vector: 32 16-byte vectors per row
     constexpr int XL = (NCT * 32 + 63) / 64;
     const int nvec = NC * 32;
-    uint4_t xv[XL], hdr, qa, qb;
-    uint32_t bias_raw;
+    uint4_t xv[XL], hdr_[RG], qa_[RG], qb_[RG];
+    uint32_t bias_raw_[RG];
     if constexpr (FAST) {
         const half_t *xg = g.X + sbi * 256;
 #pragma unroll
@@ -109,12 +112,18 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
         asm volatile("" ::: "memory");
         // 2. the block stream: a wave-uniform base plus a 32-bit lane offset
         const uint8_t *base = g.blocks + ((uint32_t)row0 * (uint32_t)g.nsb + (uint32_t)sbi) * 144u;
-        const uint32_t loff = (uint32_t)n * (uint32_t)g.nsb * 144u;
-        hdr = *(const uint4_t *)(base + loff);
-        qa = *(const uint4_t *)(base + (loff + 16u * grp) + 16);
-        qb = *(const uint4_t *)(base + (loff + 16u * grp) + 80);
-        const uint32_t bias_i = g.bias_on_rows ? (uint32_t)row0 + (t & 15) : (uint32_t)min((t >> 4) & 15, NCT - 1);
-        bias_raw = *(const uint16_t *)(g.has_bias ? (const void *)(g.bias + bias_i) : (const void *)base);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const uint32_t loff = (uint32_t)(16 * rg + n) * (uint32_t)g.nsb * 144u;
+            hdr_[rg] = *(const uint4_t *)(base + loff);
+            qa_[rg] = *(const uint4_t *)(base + (loff + 16u * grp) + 16);
+            qb_[rg] = *(const uint4_t *)(base + (loff + 16u * grp) + 80);
+        }
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const uint32_t bias_i = g.bias_on_rows ? (uint32_t)row0 + 16 * rg + (t & 15) : (uint32_t)min((t >> 4) & 15, NCT - 1);
+            bias_raw_[rg] = *(const uint16_t *)(g.has_bias ? (const void *)(g.bias + bias_i) : (const void *)base);
+        }
         asm volatile("" ::: "memory");
     } else {
         const half_t *xg = g.X + sb * g.b_bs + (int64_t)sbi * 256;
@@ -125,16 +134,25 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
         }
         asm volatile("" ::: "memory");
         // 2. the block stream: header + two 16-byte pieces of qs for row n
-        const int64_t row = min(row0 + n, g.M - 1); // rows past the end duplicate the last one; never stored
-        const uint8_t *blk = g.blocks + ((sa * g.M + row) * g.nsb + sbi) * 144;
-        hdr = *(const uint4_t *)blk;
-        qa = *(const uint4_t *)(blk + 16 + 16 * grp);
-        qb = *(const uint4_t *)(blk + 80 + 16 * grp);
+        const uint8_t *blk0 = g.blocks;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            // rows past the workgroup's or the matrix's end duplicate the last one; never stored
+            const int64_t row = min(row0 + min(16 * rg + n, g.rows_wg - 1), g.M - 1);
+            const uint8_t *blk = g.blocks + ((sa * g.M + row) * g.nsb + sbi) * 144;
+            if (rg == 0) blk0 = blk;
+            hdr_[rg] = *(const uint4_t *)blk;
+            qa_[rg] = *(const uint4_t *)(blk + 16 + 16 * grp);
+            qb_[rg] = *(const uint4_t *)(blk + 80 + 16 * grp);
+        }
         // The epilogue's bias value, fetched behind everything else so its latency is hidden.  The load is
         // unconditional (without a bias it re-reads the block header and the value is dropped): a branch
         // here makes the compiler wait for every outstanding load right after issuing this one.
-        const int64_t bias_i = g.bias_on_rows ? min(row0 + (t & 15), g.M - 1) : (int64_t)min((t >> 4) & 15, g.NC - 1);
-        bias_raw = *(const uint16_t *)(g.has_bias ? (const void *)(g.bias + bias_i) : (const void *)blk);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const int64_t bias_i = g.bias_on_rows ? min(row0 + min(16 * rg + (t & 15), g.rows_wg - 1), g.M - 1) : (int64_t)min((t >> 4) & 15, g.NC - 1);
+            bias_raw_[rg] = *(const uint16_t *)(g.has_bias ? (const void *)(g.bias + bias_i) : (const void *)blk0);
+        }
         asm volatile("" ::: "memory");
     }
 
@@ -162,92 +180,106 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     }
     asm volatile("" ::: "memory"); // the reads below are by the same wavefront; DS operations complete in order
 
-    // 4. unpack the 6-bit scales and mins (ggml get_scale_min_k4), four per dword
-    const half2_t dm = __builtin_bit_cast(half2_t, hdr[0]);
-    const float d = live ? (float)dm[0] : 0.f, dmin = live ? (float)dm[1] : 0.f;
-    const uint32_t S0 = hdr[1], S1 = hdr[2], S2 = hdr[3];
-    const uint32_t sc03 = S0 & 0x3F3F3F3Fu, mn03 = S1 & 0x3F3F3F3Fu;
-    const uint32_t sc47 = (S2 & 0x0F0F0F0Fu) | ((S0 >> 2) & 0x30303030u);
-    const uint32_t mn47 = ((S2 >> 4) & 0x0F0F0F0Fu) | ((S1 >> 2) & 0x30303030u);
-    half2_t sch[4], mnh[4];
-    q4k_bytes_to_half(sc03, sch[0], sch[1]);
-    q4k_bytes_to_half(sc47, sch[2], sch[3]);
-    q4k_bytes_to_half(mn03, mnh[0], mnh[1]);
-    q4k_bytes_to_half(mn47, mnh[2], mnh[3]);
-    auto scale_of = [&](int j) -> half_t { return sch[j >> 1][j & 1]; };
-
-    // 5. regroup so that every lane holds 8 nibbles of each of the 8 sub-blocks:
-    //    part A of a piece = sub-blocks (low, high nibbles), part B = the next two
     const int xj = min(n, NC - 1); // lanes beyond NC re-read a valid row; their outputs are dropped
     const half_t *xrow = xs + xj * XROW + q4k_x_koff(grp);
-    float4_t P = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int piece = 0; piece < 2; piece++) {
-        const uint4_t q = piece == 0 ? qa : qb;
-        auto p0 = __builtin_amdgcn_permlane32_swap(q[0], q[2], false, false);
-        auto p1 = __builtin_amdgcn_permlane32_swap(q[1], q[3], false, false);
+    for (int rg = 0; rg < RG; rg++) {
+        const uint4_t hdr = hdr_[rg], qa = qa_[rg], qb = qb_[rg];
+        // 4. unpack the 6-bit scales and mins (ggml get_scale_min_k4), four per dword
+        const half2_t dm = __builtin_bit_cast(half2_t, hdr[0]);
+        const float d = live ? (float)dm[0] : 0.f, dmin = live ? (float)dm[1] : 0.f;
+        const uint32_t S0 = hdr[1], S1 = hdr[2], S2 = hdr[3];
+        const uint32_t sc03 = S0 & 0x3F3F3F3Fu, mn03 = S1 & 0x3F3F3F3Fu;
+        const uint32_t sc47 = (S2 & 0x0F0F0F0Fu) | ((S0 >> 2) & 0x30303030u);
+        const uint32_t mn47 = ((S2 >> 4) & 0x0F0F0F0Fu) | ((S1 >> 2) & 0x30303030u);
+        half2_t sch[4], mnh[4];
+        q4k_bytes_to_half(sc03, sch[0], sch[1]);
+        q4k_bytes_to_half(sc47, sch[2], sch[3]);
+        q4k_bytes_to_half(mn03, mnh[0], mnh[1]);
+        q4k_bytes_to_half(mn47, mnh[2], mnh[3]);
+        auto scale_of = [&](int j) -> half_t { return sch[j >> 1][j & 1]; };
+
+        // 5. regroup so that every lane holds 8 nibbles of each of the 8 sub-blocks:
+        //    part A of a piece = sub-blocks (low, high nibbles), part B = the next two
+        float4_t P = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int part = 0; part < 2; part++) {
-            const uint32_t v0 = p0[part], v1 = p1[part];
-            const int jlo = piece * 4 + part * 2, jhi = jlo + 1; // sub-blocks of the low / high nibbles
-            const half8_t blo = q4k_scaled(v0 & 0x0F0F0F0Fu, v1 & 0x0F0F0F0Fu, scale_of(jlo));
-            const half8_t bhi = q4k_scaled((v0 >> 4) & 0x0F0F0F0Fu, (v1 >> 4) & 0x0F0F0F0Fu, scale_of(jhi));
-            const half8_t alo = __builtin_bit_cast(half8_t, *(const uint4_t *)(xrow + 32 * jlo));
-            const half8_t ahi = __builtin_bit_cast(half8_t, *(const uint4_t *)(xrow + 32 * jhi));
-            P = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, blo, P, 0, 0, 0);
-            P = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi, P, 0, 0, 0);
+        for (int piece = 0; piece < 2; piece++) {
+            const uint4_t q = piece == 0 ? qa : qb;
+            auto p0 = __builtin_amdgcn_permlane32_swap(q[0], q[2], false, false);
+            auto p1 = __builtin_amdgcn_permlane32_swap(q[1], q[3], false, false);
+#pragma unroll
+            for (int part = 0; part < 2; part++) {
+                const uint32_t v0 = p0[part], v1 = p1[part];
+                const int jlo = piece * 4 + part * 2, jhi = jlo + 1; // sub-blocks of the low / high nibbles
+                const half8_t blo = q4k_scaled(v0 & 0x0F0F0F0Fu, v1 & 0x0F0F0F0Fu, scale_of(jlo));
+                const half8_t bhi = q4k_scaled((v0 >> 4) & 0x0F0F0F0Fu, (v1 >> 4) & 0x0F0F0F0Fu, scale_of(jhi));
+                const half8_t alo = __builtin_bit_cast(half8_t, *(const uint4_t *)(xrow + 32 * jlo));
+                const half8_t ahi = __builtin_bit_cast(half8_t, *(const uint4_t *)(xrow + 32 * jhi));
+                P = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, blo, P, 0, 0, 0);
+                P = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi, P, 0, 0, 0);
+            }
         }
-    }
-    // 6. the min term: K slots 0..7 = high parts of the 8 sub-block sums, 8..15 = low parts, rest zero
-    half8_t bm = {mnh[0][0], mnh[0][1], mnh[1][0], mnh[1][1], mnh[2][0], mnh[2][1], mnh[3][0], mnh[3][1]};
-    if (grp >= 2) bm = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    const half8_t am = __builtin_bit_cast(half8_t, *(const uint4_t *)(sxs + xj * 16 + 8 * (grp & 1)));
-    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-    const float4_t T = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm, zero, 0, 0, 0);
-    // a lane's result register r is activation vector 4 * grp + r: only those that exist are summed
-    constexpr int NR = NCT < 4 ? NCT : 4;
-    if (NCT >= 16 || 4 * grp < NCT) {
+        // 6. the min term: K slots 0..7 = high parts of the 8 sub-block sums, 8..15 = low parts, rest zero
+        half8_t bm = {mnh[0][0], mnh[0][1], mnh[1][0], mnh[1][1], mnh[2][0], mnh[2][1], mnh[3][0], mnh[3][1]};
+        if (grp >= 2) bm = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        const half8_t am = __builtin_bit_cast(half8_t, *(const uint4_t *)(sxs + xj * 16 + 8 * (grp & 1)));
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        const float4_t T = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm, zero, 0, 0, 0);
+        // a lane's result register r is activation vector 4 * grp + r: only those that exist are summed
+        constexpr int NR = NCT < 4 ? NCT : 4;
+        if (NCT >= 16 || 4 * grp < NCT) {
 #pragma unroll
-        for (int r = 0; r < NR; r++) psum[wave * 256 + (4 * grp + r) * 16 + n] = fmaf(-dmin, T[r], d * P[r]);
+            for (int r = 0; r < NR; r++) psum[(wave * RG + rg) * 256 + (4 * grp + r) * 16 + n] = fmaf(-dmin, T[r], d * P[r]);
+        }
     }
 
     // 7. sum the K slices
     __syncthreads();
     if (t < 16 * NCT) {
-        float v = 0.f;
-        for (int w2 = 0; w2 < nwaves; w2++) v += psum[w2 * 256 + t];
         const int j = t >> 4;
-        const int64_t i = row0 + (t & 15);
-        if (FAST || (j < g.NC && i < g.M)) g.out[s * g.o_bs + i * g.o_is + j * g.o_js] = (half_t)rt_act(v + (g.has_bias ? (float)__builtin_bit_cast(half2_t, bias_raw)[0] : 0.f), g.act);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            float v = 0.f;
+            for (int w2 = 0; w2 < nwaves; w2++) v += psum[(w2 * RG + rg) * 256 + t];
+            const int64_t i = row0 + 16 * rg + (t & 15);
+            if (FAST || (j < g.NC && i < g.M && 16 * rg + (t & 15) < g.rows_wg))
+                g.out[s * g.o_bs + i * g.o_is + j * g.o_js] = (half_t)rt_act(v + (g.has_bias ? (float)__builtin_bit_cast(half2_t, bias_raw_[rg])[0] : 0.f), g.act);
+        }
     }
 }
 
-template <int NCT, bool FAST>
+template <int NCT, bool FAST, int RG>
 static hipError_t launch_q4k_kernel(dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvQ4kArgs &g) {
     if (lds > 48 * 1024) {
-        const hipError_t e = ensure_lds_limit<&gemv_q4k_mfma_kernel<NCT, FAST>>();
+        const hipError_t e = ensure_lds_limit<&gemv_q4k_mfma_kernel<NCT, FAST, RG>>();
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<NCT, FAST>), grid, dim3(nwaves * 64), lds, st, g);
+    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<NCT, FAST, RG>), grid, dim3(nwaves * 64), lds, st, g);
     return hipGetLastError();
 }
 
 template <int NCT>
-static hipError_t launch_q4k_one(dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvQ4kArgs &g) {
-    const bool regular = grid.y == 1 && g.a_stack == 1 && g.b_stack == 1 && g.M % 16 == 0 && g.NC == NCT &&
-                         g.nsb == nwaves && g.M * g.nsb * 144 < (int64_t(1) << 31) &&
+static hipError_t launch_q4k_one(int rg, dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvQ4kArgs &g) {
+    const bool regular = grid.y == 1 && g.a_stack == 1 && g.b_stack == 1 && g.M % (16 * rg) == 0 && g.rows_wg == 16 * rg &&
+                         g.NC == NCT && g.nsb == nwaves && g.M * g.nsb * 144 < (int64_t(1) << 31) &&
                          (int64_t)g.NC * g.b_js < (int64_t(1) << 30);
-    if (regular) return launch_q4k_kernel<NCT, true>(grid, nwaves, lds, st, g);
-    return launch_q4k_kernel<NCT, false>(grid, nwaves, lds, st, g);
+    if constexpr (NCT == 16) { // two row groups are only dealt where 9..16 vectors leave room for one workgroup per compute unit
+        if (rg == 2) return regular ? launch_q4k_kernel<NCT, true, 2>(grid, nwaves, lds, st, g) : launch_q4k_kernel<NCT, false, 2>(grid, nwaves, lds, st, g);
+    }
+    if (rg != 1) return hipErrorInvalidValue;
+    if (regular) return launch_q4k_kernel<NCT, true, 1>(grid, nwaves, lds, st, g);
+    return launch_q4k_kernel<NCT, false, 1>(grid, nwaves, lds, st, g);
 }
 
 // Tunable: non-zero keeps Q4_K weights off this kernel (for comparisons).
 RT_TUNABLE(g_gemv_q4k_disable_mfma, 0);
+// Tunable: 1 or 2 forces that many 16-row groups per workgroup (0 = by residency, see the launcher).
+RT_TUNABLE(g_gemv_q4k_mfma_rg, 0);
 
 // Q4_K weights, f16 activations, 1..16 vectors, K a multiple of 256 and at most 4096.
 // hipErrorNotSupported means another kernel must run.
 hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, const void *bias, void *out,
-                                hipStream_t stream, const DeviceInfo &) {
+                                hipStream_t stream, const DeviceInfo &dev) {
     if (g_gemv_q4k_disable_mfma) return hipErrorNotSupported;
     if (p.a_dt != RT_Q4_K || p.act_dt != RT_F16 || p.N < 1 || p.N > 16 || p.K % 256 != 0 || p.K < 256 || p.K > 4096)
         return hipErrorNotSupported;
@@ -263,16 +295,27 @@ hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, 
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
     if (p.has_bias && ((uintptr_t)bias & 1u)) return hipErrorNotSupported;
     const int nwaves = g.nsb < 4 ? 4 : g.nsb; // the final sum uses 256 threads
-    const size_t lds = (size_t)nwaves * g.NC * (256 + kQ4kXPad + 16) * 2 + (size_t)nwaves * 1024;
+    // Rows per workgroup: 16, unless the activations' LDS (9..16 vectors) leaves one workgroup per compute unit and
+    // the 16-row workgroups would run in rounds; then every compute unit gets one workgroup with its share of the
+    // rows, up to 32 (8192 rows, 16 vectors: 512 workgroups in two rounds 9.3 us -> 256 in one 7.7 us).
+    const size_t lds_x = (size_t)nwaves * g.NC * (256 + kQ4kXPad + 16) * 2;
+    int rg = 1, rows_wg = 16;
+    if (g.NC > 8 && p.stacks == 1 && 2 * (lds_x + (size_t)nwaves * 1024) > 160 * 1024 && (p.M + 15) / 16 > dev.num_cus) {
+        const int64_t per = ((p.M + dev.num_cus - 1) / dev.num_cus + 7) & ~(int64_t)7;
+        if (per <= 32) rows_wg = (int)per, rg = (rows_wg + 15) / 16;
+    }
+    if (g_gemv_q4k_mfma_rg > 0 && g.NC > 8) rg = g_gemv_q4k_mfma_rg, rows_wg = 16 * rg;
+    g.rows_wg = rows_wg;
+    const size_t lds = lds_x + (size_t)nwaves * rg * 1024;
     if (lds > 160 * 1024) return hipErrorNotSupported;
-    const int64_t groups = (p.M + 15) / 16;
+    const int64_t groups = (p.M + rows_wg - 1) / rows_wg;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
-    if (g.NC <= 1) return launch_q4k_one<1>(grid, nwaves, lds, stream, g);
-    if (g.NC <= 2) return launch_q4k_one<2>(grid, nwaves, lds, stream, g);
-    if (g.NC <= 4) return launch_q4k_one<4>(grid, nwaves, lds, stream, g);
-    if (g.NC <= 8) return launch_q4k_one<8>(grid, nwaves, lds, stream, g);
-    return launch_q4k_one<16>(grid, nwaves, lds, stream, g);
+    if (g.NC <= 1) return launch_q4k_one<1>(rg, grid, nwaves, lds, stream, g);
+    if (g.NC <= 2) return launch_q4k_one<2>(rg, grid, nwaves, lds, stream, g);
+    if (g.NC <= 4) return launch_q4k_one<4>(rg, grid, nwaves, lds, stream, g);
+    if (g.NC <= 8) return launch_q4k_one<8>(rg, grid, nwaves, lds, stream, g);
+    return launch_q4k_one<16>(rg, grid, nwaves, lds, stream, g);
 }
 
 } // namespace rt

@@ -378,6 +378,31 @@ def test_q4k_streaming_shapes(device, oracle):
     check(oracle, got, want, DType.F16, "no trans_out")
 
 
+def test_q4k_streaming_rows_dealt_one_workgroup_per_compute_unit(device, oracle):
+    """With 9..16 vectors and K from 2560 one workgroup of the Q4_K streaming kernel fits a compute unit; more than
+    256 of the 16-row workgroups would run in rounds, so every compute unit gets one workgroup of up to 32 rows:
+    whole double groups (8192 rows), a half-empty second group (4104 rows: 24 per workgroup), and a row count
+    whose share is above 32 (back to 16-row workgroups); then one-hot activations, bit for bit."""
+    for i, (M, N, K) in enumerate([(16, 8192, 3072), (13, 4104, 2560), (16, 8200, 2560)]):
+        rng = np.random.default_rng(490 + i)
+        blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+        x = rng.standard_normal((1, M, K)).astype(np.float16)
+        for to in (True, False):
+            bias = rng.standard_normal(N if to else M).astype(np.float16)
+            got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (N, K)), Tensor.from_data(x),
+                             Tensor.from_data(bias), False, True, to)
+            want = oracle.matmul_ref(blocks, oracle.Q4_K, (N, K), x, oracle.F16, x.shape, bias, False, True, to)
+            check(oracle, got, want, DType.F16, (M, N, K, to))
+    N, K = 4104, 2560
+    blocks = oracle.q4k_quantize((np.random.default_rng(495).standard_normal((N, K)) * 0.02).astype(np.float32))
+    dq = oracle.q4k_dequantize(blocks).reshape(N, K)
+    cols = np.arange(16) * 157 + 3
+    x = np.zeros((16, K), dtype=np.float16)
+    x[np.arange(16), cols] = 1
+    got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (N, K)), Tensor.from_data(x), None, False, True, True)
+    assert np.array_equal(got, dq[:, cols].T.astype(np.float16))
+
+
 def test_q4k_row_streaming_long_rows(device, oracle):
     """Q4_K weights with K above 4096 against one vector take the row-streaming kernel (a wavefront per row, the
     row read as a run of 16-byte vectors, block headers handed to the lanes of their blocks through LDS): K from
