@@ -728,6 +728,222 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_q8dl_kernel(Gemm
     nt_epilogue<TM, TN, WM, WN>(g, acc, smem, s, i0, j0, wi, wj, wave, lane);
 }
 
+// ---------------------------------------------------------------------------
+// Q8_0H x f16 with the widening done by the loading wavefronts.  In gemm_nt_q8dl_kernel the four
+// multiplying wavefronts also turn every code fragment they read into f16 (50 of their 153 vector
+// instructions per K step) while the loading wavefronts' vector units idle.  Here LW = 4 loading
+// wavefronts, one per SIMD, fetch the int8 tile into registers (a lane: 16 codes of one row), widen it
+// (exact) and store f16 code tiles into the ring in the f16 kernel's swizzled layout; the activation tile still
+// goes global -> LDS directly.  The multiplying wavefronts then run the f16 kernel's fragment reads and,
+// per block of 32, one MFMA from zero whose four sums per lane are folded into the accumulators with the
+// block's f16 scale two MFMAs later, as before: no weight is rounded.
+//
+// Ring of four stages of (BM + BN) x 64 halves.  Loading wavefront, iteration j: request the codes of tile
+// j + 3 (registers, set (j + 3) % 4) and its activation rows (LDS-DMA into stage (j + 3) % 4, last read
+// before the barrier that ended iteration j - 1); wait for the codes of tile j + 1, requested two
+// iterations ago (everything older has landed with them, the activation rows of tile j + 1 included);
+// widen and store them into stage (j + 1) % 4; barrier.  Requires K % 256 == 0 (scales in groups of 8).
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int LW>
+__global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_q8w_kernel(GemmNtArgs g) {
+    constexpr int STAGES = 4, AHEAD = 2;
+    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
+    constexpr int STAGE_HALFS = (BM + BN) * NT_LDK;
+    constexpr int NREAD = TM + TN;
+    static_assert(BM % 16 == 0 && BN % (8 * LW) == 0, "tile rows must fill whole chunks");
+    static_assert(TM * TN >= NREAD, "not enough MFMAs to spread the reads over");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    half_t *ring = (half_t *)smem; // [STAGES][BM + BN][64]
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+
+    int64_t ti, tj;
+    nt_tile_of(blockIdx.x, g.tiles_i, g.tiles_j, ti, tj); // XCD-aware tile order (see the file comment)
+    const int64_t i0 = ti * BM, j0 = tj * BN;
+    const int64_t s = blockIdx.y;
+    const int64_t kbase = (int64_t)blockIdx.z * g.k_len; // this workgroup's share of K (all of it without a split)
+    const int64_t a_el = (g.a_stack == 1 ? 0 : s) * g.a_bs + kbase, b_el = (g.b_stack == 1 ? 0 : s) * g.b_bs + kbase;
+    const int64_t nk = g.k_len / NT_BK; // a multiple of 4
+
+    if (wave >= 4) {
+        const int lw = wave - 4;
+        constexpr int ACH = BM / 16;            // 16-row pieces of the code tile (one load instruction each)
+        constexpr int NA = (ACH + LW - 1) / LW; // per loading wavefront
+        constexpr int LCHB = BN / 8 / LW;       // 8-row chunks of the activation tile per loading wavefront
+        static_assert(AHEAD * (LCHB + NA) < 64, "the wait counter has six bits");
+        const uint8_t *ga[NA];
+        int adst[NA]; // this lane's row within the code tile
+        bool alive[NA];
+        const int piece = lane & 3;
+#pragma unroll
+        for (int c = 0; c < NA; c++) {
+            const int ch = lw + c * LW;
+            alive[c] = ch < ACH; // wave-uniform
+            const int row = min(ch, ACH - 1) * 16 + (lane >> 2);
+            ga[c] = (const uint8_t *)g.A + a_el + min(i0 + row, g.M - 1) * g.a_rs + 16 * piece;
+            adst[c] = row;
+        }
+        const half_t *gb[LCHB];
+#pragma unroll
+        for (int c = 0; c < LCHB; c++) {
+            const int row = (lw + c * LW) * 8 + (lane >> 3);
+            const int kv = (lane & 7) ^ ((row >> 1) & 7);
+            gb[c] = g.B + b_el + min(j0 + row, g.N - 1) * g.b_js + 8 * kv;
+        }
+        uint4_t ra[STAGES][NA];
+        auto request = [&](int slot, int64_t tile) __attribute__((always_inline)) {
+            const int64_t k0 = min(tile, nk - 1) * NT_BK; // past the last tile: re-read it, never used
+            half_t *st = ring + slot * STAGE_HALFS + BM * NT_LDK;
+#pragma unroll
+            for (int c = 0; c < LCHB; c++)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb[c] + k0),
+                                                 (__attribute__((address_space(3))) void *)(st + (lw + c * LW) * 8 * NT_LDK), 16, 0, 0);
+#pragma unroll
+            for (int c = 0; c < NA; c++) ra[slot][c] = *(const uint4_t *)(ga[c] + k0);
+        };
+        auto widen_store = [&](int slot) __attribute__((always_inline)) {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0x0F70 | ((AHEAD * (LCHB + NA)) & 0xF) | ((((AHEAD * (LCHB + NA)) >> 4) & 0x3) << 14));
+            half_t *st = ring + slot * STAGE_HALFS;
+#pragma unroll
+            for (int c = 0; c < NA; c++) {
+                if (alive[c]) {
+                    half2_t h[8];
+#pragma unroll
+                    for (int d = 0; d < 4; d++) nt_cvt_i8x4(ra[slot][c][d], h[2 * d], h[2 * d + 1]);
+                    const uint4_t lo = {__builtin_bit_cast(uint32_t, h[0]), __builtin_bit_cast(uint32_t, h[1]),
+                                        __builtin_bit_cast(uint32_t, h[2]), __builtin_bit_cast(uint32_t, h[3])};
+                    const uint4_t hi = {__builtin_bit_cast(uint32_t, h[4]), __builtin_bit_cast(uint32_t, h[5]),
+                                        __builtin_bit_cast(uint32_t, h[6]), __builtin_bit_cast(uint32_t, h[7])};
+                    *(uint4_t *)(st + nt_slot(adst[c], 2 * piece)) = lo;
+                    *(uint4_t *)(st + nt_slot(adst[c], 2 * piece + 1)) = hi;
+                }
+            }
+        };
+        auto publish = [&]() __attribute__((always_inline)) {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the widened tile is in LDS
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        };
+        request(0, 0);
+        request(1, 1);
+        request(2, 2);
+        widen_store(0);
+        publish(); // tile 0
+        for (int64_t kg = 0; kg < nk; kg += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                request((u + 3) & 3, kg + u + 3); // into the stage that was read for the last time before the barrier of iteration kg + u - 1
+                widen_store((u + 1) & 3);         // tile kg + u + 1
+                publish();
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): nothing may land once the epilogue reuses the ring
+        __syncthreads();
+        return;
+    }
+
+    // ---- multiplying wavefronts: the f16 kernel's fragments, the Q8 fold
+    const int wi = wave >> 1, wj = wave & 1;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int swz = (fr >> 1) & 7;
+    // this lane's scale rows: 16 bytes = the 8 blocks of four K tiles
+    const half_t *sp[TM];
+#pragma unroll
+    for (int a = 0; a < TM; a++) {
+        const int64_t gr = min(i0 + wi * WM + a * 16 + fr, g.M - 1);
+        sp[a] = g.scales + ((a_el + gr * g.a_rs) >> 5);
+    }
+    struct Frags {
+        half8_t a[TM], b[TN];
+    };
+    auto read_one = [&](int stage, int kk, Frags &f, int i) {
+        const half_t *as = ring + stage * STAGE_HALFS + (wi * WM + fr) * NT_LDK + (((kk * 4 + fg) ^ swz) << 3);
+        const half_t *bs = ring + stage * STAGE_HALFS + BM * NT_LDK + (wj * WN + fr) * NT_LDK + (((kk * 4 + fg) ^ swz) << 3);
+        if (i < TM)
+            f.a[i] = __builtin_bit_cast(half8_t, *(const uint4_t *)(as + i * 16 * NT_LDK));
+        else
+            f.b[i - TM] = __builtin_bit_cast(half8_t, *(const uint4_t *)(bs + (i - TM) * 16 * NT_LDK));
+    };
+    uint4_t sc_cur[TM], sc_nxt[TM];
+#pragma unroll
+    for (int a = 0; a < TM; a++) sc_cur[a] = *(const uint4_t *)sp[a];
+    auto next_tile = [&]() {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this tile's fragment reads have returned
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    next_tile(); // tile 0
+
+    Frags r0, r1;
+#pragma unroll
+    for (int i = 0; i < NREAD; i++) read_one(0, 0, r0, i);
+    int cur = 0, nxt = 1;
+    auto scale_of = [&](int a, int blk) -> half_t { return __builtin_bit_cast(half8_t, sc_cur[a])[blk]; };
+    float accs[TM][TN][4]; // the accumulators as scalars: each is written by a vector instruction of its own
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) accs[a][b][r] = 0.f;
+    // One K step (a block of 32): TM * TN MFMAs on the fragments in `rc` from zero, each folded into the
+    // accumulators two MFMAs later with the scale of block `blk`; between them the fragment reads of the
+    // following K step into `rn`.
+    auto k_step = [&](const Frags &rc, Frags &rn, int blk, int rstage, int rkk) {
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        float4_t P[3]; // partial sums of three tiles in flight: a tile is folded two MFMAs after its own
+        int slot = 0;
+#pragma unroll
+        for (int idx = 0; idx < TM * TN + 2; idx++) {
+            const int a = idx / TN, b = idx % TN;
+            if (idx < TM * TN) {
+                P[idx % 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(rc.b[b], rc.a[a], zero, 0, 0, 0);
+                asm volatile("" : "+v"(P[idx % 3])); // instruction selection lets results nobody orders float: this MFMA is issued here
+                if (slot < NREAD) read_one(rstage, rkk, rn, slot++); // the fragments of the following K step
+            }
+            if (idx >= 2) {
+                const int fa = (idx - 2) / TN, fb = (idx - 2) % TN;
+                const float d = (float)scale_of(fa, blk);
+#pragma unroll
+                for (int r = 0; r < 4; r++) accs[fa][fb][r] = fmaf(d, P[(idx - 2) % 3][r], accs[fa][fb][r]);
+                // ... and the sums are folded here, not gathered at the end of the loop body with every partial sum kept alive
+                asm volatile("" : "+v"(accs[fa][fb][0]), "+v"(accs[fa][fb][1]), "+v"(accs[fa][fb][2]), "+v"(accs[fa][fb][3]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int64_t kg = 0; kg < nk; kg += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (u == 0) {
+                // scales of the next group of four tiles, a group ahead of their use
+                const int64_t gn = min(kg + 4, nk - 4) >> 2;
+#pragma unroll
+                for (int a = 0; a < TM; a++) sc_nxt[a] = *(const uint4_t *)(sp[a] + 8 * gn);
+            }
+            k_step(r0, r1, 2 * u, cur, 1);
+            next_tile();
+            k_step(r1, r0, 2 * u + 1, nxt, 0);
+            cur = nxt;
+            nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
+        }
+#pragma unroll
+        for (int a = 0; a < TM; a++) sc_cur[a] = sc_nxt[a];
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
+    float4_t acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++) acc[a][b] = float4_t{accs[a][b][0], accs[a][b][1], accs[a][b][2], accs[a][b][3]};
+    nt_epilogue<TM, TN, WM, WN>(g, acc, smem, s, i0, j0, wi, wj, wave, lane);
+}
+
 // Second pass of a split-K launch: out = round(act(sum over the splits + bias)).  One thread per four
 // consecutive i (the partial sums' contiguous axis); M need not be a multiple of four.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmNtArgs g) {
@@ -778,6 +994,16 @@ static hipError_t launch_nt_q8dl(const GemmNtArgs &g, int64_t stacks, hipStream_
     if (const hipError_t e = ensure_lds_limit<&gemm_nt_q8dl_kernel<BM, BN, STAGES, LW>>(); e != hipSuccess) return e;
     dim3 grid((unsigned)((int64_t)g.tiles_i * g.tiles_j), (unsigned)stacks, (unsigned)g.ksplit);
     hipLaunchKernelGGL((gemm_nt_q8dl_kernel<BM, BN, STAGES, LW>), grid, dim3(NT_THREADS + 64 * LW), lds, st, g);
+    if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    return g.ksplit > 1 ? launch_splitk_reduce(g, stacks, st) : hipSuccess;
+}
+
+template <int BM, int BN, int LW>
+static hipError_t launch_nt_q8w(const GemmNtArgs &g, int64_t stacks, hipStream_t st) {
+    const size_t lds = (size_t)4 * (BM + BN) * NT_LDK * 2;
+    if (const hipError_t e = ensure_lds_limit<&gemm_nt_q8w_kernel<BM, BN, LW>>(); e != hipSuccess) return e;
+    dim3 grid((unsigned)((int64_t)g.tiles_i * g.tiles_j), (unsigned)stacks, (unsigned)g.ksplit);
+    hipLaunchKernelGGL((gemm_nt_q8w_kernel<BM, BN, LW>), grid, dim3(NT_THREADS + 64 * LW), lds, st, g);
     if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     return g.ksplit > 1 ? launch_splitk_reduce(g, stacks, st) : hipSuccess;
 }
@@ -912,6 +1138,8 @@ static hipError_t launch_nt(const GemmNtArgs &g, int64_t stacks, hipStream_t st)
 
 // Tunable: 0 = automatic, 1 = never take this kernel (for comparisons).
 RT_TUNABLE(g_gemm_nt_disable, 0);
+// Tunable: 1 = Q8_0H tiles widened by the multiplying wavefronts (gemm_nt_q8dl_kernel) instead of the loading ones.
+RT_TUNABLE(g_gemm_nt_q8_variant, 0);
 
 // f16 or Q8_0H A with K-contiguous rows, f16 B with K-contiguous rows.
 // hipErrorNotSupported: the problem does not fit; the generic tiled GEMM runs instead.
@@ -1025,7 +1253,7 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
                                      : launch_nt_dl<BM, BN, 3, 2>(g, p.stacks, stream);
     }
     if (dl_q8)
-        return launch_nt_q8dl<BM, BN, 4, 2>(g, p.stacks, stream);
+        return g_gemm_nt_q8_variant == 1 ? launch_nt_q8dl<BM, BN, 4, 2>(g, p.stacks, stream) : launch_nt_q8w<BM, BN, 4>(g, p.stacks, stream);
     if (q8) return kfull ? launch_nt<BM, BN, true, true>(g, p.stacks, stream) : launch_nt<BM, BN, true, false>(g, p.stacks, stream);
     return kfull ? launch_nt<BM, BN, false, true>(g, p.stacks, stream) : launch_nt<BM, BN, false, false>(g, p.stacks, stream);
 }
