@@ -6,8 +6,8 @@
 //                          directly into a ring of stages by two wavefronts that do nothing else,
 //                          issue order pinned (the fast path for the Phi-2 prefill shape:
 //                          10240 x 512 outputs = 256 workgroups, one per CU)
-//   gemm_nt_q8dl_kernel    Q8_0H x f16, K % 256 == 0: the same pipeline with int8 tiles in LDS; the codes
-//                          become f16 integers at read time, each block of 32 is multiplied from zero and
+//   gemm_nt_q8w_kernel     Q8_0H x f16, K % 256 == 0: the same pipeline; four loading wavefronts widen the int8
+//                          tile to f16 codes on its way into LDS, each block of 32 is multiplied from zero and
 //                          its partial sums are folded into the accumulators with the block's scale in f32
 //   gemm_nt_shortk_kernel  f16 x f16, K <= 128 (attention scores): a resident strip of B rows,
 //                          A tiles prefetched through registers, output written as it is produced
@@ -519,224 +519,18 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
 }
 
 // ---------------------------------------------------------------------------
-// Q8_0H x f16 variant with direct-to-LDS loads.  The int8 codes travel global -> LDS
-// untouched (64 bytes per row and K tile, half the f16 traffic); a wavefront turns them into
-// f16 integers (exact) when it reads its fragments and multiplies those: one MFMA per tile
-// and block of 32 from a zero accumulator, whose four partial sums per lane are then
-// folded into the f32 accumulators with the block's scale (v_fma_mix: the f16 scale is an
-// operand as it is).  No weight is rounded.  An earlier version made the operand q * d
-// itself, exactly, as the sum of two f16 (hi = rn(q * d), lo = fma(q, d, -hi)) and took two
-// MFMAs per tile into the running accumulator: 64.5 us at [512 x 2560] . [10240 x 2560]^T
-// where this one takes 51; the second MFMA cost more than the 80 fused multiply-adds do.
-//
-// LDS A tile: row r holds its eight 8-byte slots s at s ^ (((r >> 2) & 3) << 1): a lane
-// group's 16 rows x 8 bytes (one fragment read) and a load instruction's 16 rows x 64
-// bytes both spread over all banks.  The scales of a lane's rows are fetched straight
-// into registers, 8 blocks (four K tiles) per 16-byte load, one group ahead.
-// Requires K % 256 == 0.
-// ---------------------------------------------------------------------------
-// The tile loads are issued by LW wavefronts of their own (as in gemm_nt_dl_kernel); the four
-// multiplying wavefronts issue no tile load.
-template <int BM, int BN, int STAGES, int LW>
-__global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_q8dl_kernel(GemmNtArgs g) {
-    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 16, TN = WN / 16;
-    constexpr int A_CHT = BM / 16;            // 16-row chunks of the int8 A tile (1 KiB each)
-    static_assert(LW > 0 && BM % 32 == 0 && BN % 32 == 0, "tile rows must fill whole chunks");
-    constexpr int A_BYTES = BM * NT_BK, STAGE_BYTES = A_BYTES + BN * NT_LDK * 2;
-    constexpr int NREAD = TM + TN;
-    static_assert(TM * TN >= NREAD, "not enough MFMAs to spread the reads over");
-
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int t = threadIdx.x, lane = t & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wi = wave >> 1, wj = wave & 1;
-    const int fr = lane & 15, fg = lane >> 4;
-
-    int64_t ti, tj;
-    nt_tile_of(blockIdx.x, g.tiles_i, g.tiles_j, ti, tj); // XCD-aware tile order (see the file comment)
-    const int64_t i0 = ti * BM, j0 = tj * BN;
-    const int64_t s = blockIdx.y;
-    const int64_t kbase = (int64_t)blockIdx.z * g.k_len; // this workgroup's share of K (all of it without a split)
-    const int64_t a_el = (g.a_stack == 1 ? 0 : s) * g.a_bs + kbase, b_el = (g.b_stack == 1 ? 0 : s) * g.b_bs + kbase;
-
-    if constexpr (LW > 0) {
-        if (wave >= 4) {
-            // ---- loading wavefront: the tile's 1 KiB chunks (A_CHT of 16 int8 rows, then BN / 8 of 8 f16
-            // rows), dealt round-robin; layouts and swizzles as described for the other wavefronts below
-            constexpr int CH = A_CHT + BN / 8, LCH = (CH + LW - 1) / LW;
-            static_assert(CH % LW == 0 && (STAGES - 2) * LCH < 64, "chunks must deal out evenly; the wait counter has six bits");
-            const int lw = wave - 4;
-            const uint8_t *gp[LCH];
-            int kmul[LCH], dst[LCH]; // bytes per element of K; byte offset of the chunk within a stage
-#pragma unroll
-            for (int c = 0; c < LCH; c++) {
-                const int ch = lw + c * LW;
-                if (ch < A_CHT) {
-                    const int row = ch * 16 + (lane >> 2);
-                    const int piece = (lane & 3) ^ ((row >> 2) & 3);
-                    gp[c] = (const uint8_t *)g.A + a_el + min(i0 + row, g.M - 1) * g.a_rs + 16 * piece;
-                    kmul[c] = 1, dst[c] = ch * 16 * NT_BK;
-                } else {
-                    const int cb = ch - A_CHT, row = cb * 8 + (lane >> 3);
-                    const int kv = (lane & 7) ^ ((row >> 1) & 7);
-                    gp[c] = (const uint8_t *)(g.B + b_el + min(j0 + row, g.N - 1) * g.b_js + 8 * kv);
-                    kmul[c] = 2, dst[c] = A_BYTES + cb * 8 * NT_LDK * 2;
-                }
-            }
-            auto issue_tile = [&](int stage, int64_t k0) {
-                uint8_t *st = smem + stage * STAGE_BYTES;
-#pragma unroll
-                for (int c = 0; c < LCH; c++)
-                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gp[c] + k0 * kmul[c]),
-                                                     (__attribute__((address_space(3))) void *)(st + dst[c]), 16, 0, 0);
-            };
-            constexpr int kKeep = (STAGES - 2) * LCH;
-            auto publish = [&]() {
-                asm volatile("" ::: "memory");
-                __builtin_amdgcn_s_waitcnt(0x0F70 | (kKeep & 0xF) | (((kKeep >> 4) & 0x3) << 14));
-                __builtin_amdgcn_s_barrier();
-                asm volatile("" ::: "memory");
-            };
-            const int64_t nkl = g.k_len / NT_BK;
-#pragma unroll
-            for (int st = 0; st < STAGES - 1; st++) issue_tile(st, min<int64_t>(st, nkl - 1) * NT_BK);
-            publish(); // tile 0
-            int wrl = STAGES - 1;
-            for (int64_t kt = 0; kt < nkl; kt++) {
-                issue_tile(wrl, min(kt + STAGES - 1, nkl - 1) * NT_BK);
-                publish(); // tile kt + 1
-                wrl = wrl + 1 == STAGES ? 0 : wrl + 1;
-            }
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            __syncthreads();
-            return;
-        }
-    }
-
-    // this lane's scale rows: 16 bytes = the 8 blocks of four K tiles
-    const half_t *sp[TM];
-#pragma unroll
-    for (int a = 0; a < TM; a++) {
-        const int64_t gr = min(i0 + wi * WM + a * 16 + fr, g.M - 1);
-        sp[a] = g.scales + ((a_el + gr * g.a_rs) >> 5);
-    }
-
-    // fragment reads: raw A codes (8 bytes) and B vectors (16 bytes)
-    const int a_swz = ((fr >> 2) & 3) << 1, b_swz = (fr >> 1) & 7;
-    struct Raw {
-        uint2_t a[TM];
-        half8_t b[TN];
-    };
-    auto read_one = [&](int stage, int kk, Raw &f, int i) {
-        const uint8_t *as = smem + stage * STAGE_BYTES;
-        if (i < TM) {
-            f.a[i] = *(const uint2_t *)(as + (wi * WM + i * 16 + fr) * NT_BK + (((kk * 4 + fg) ^ a_swz) << 3));
-        } else {
-            const half_t *bs = (const half_t *)(as + A_BYTES) + (wj * WN + fr) * NT_LDK + (((kk * 4 + fg) ^ b_swz) << 3);
-            f.b[i - TM] = __builtin_bit_cast(half8_t, *(const uint4_t *)(bs + (i - TM) * 16 * NT_LDK));
-        }
-    };
-    const int64_t nk = g.k_len / NT_BK; // a multiple of 4
-    uint4_t sc_cur[TM], sc_nxt[TM];
-#pragma unroll
-    for (int a = 0; a < TM; a++) sc_cur[a] = *(const uint4_t *)sp[a];
-    // The tile's LDS reads are done (the scale loads are waited for where they are used); past the barrier
-    // the next tile, whose loads the loading wavefronts have waited for, is whole.
-    auto next_tile = [&]() {
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-    };
-    next_tile(); // tile 0
-
-    Raw r0, r1;
-#pragma unroll
-    for (int i = 0; i < NREAD; i++) read_one(0, 0, r0, i);
-    int cur = 0, nxt = 1;
-    // scale of row fragment a for block `blk` (0..7) of the current group of four tiles
-    auto scale_of = [&](int a, int blk) -> half_t { return __builtin_bit_cast(half8_t, sc_cur[a])[blk]; };
-    // One K step (a block of 32): TM * TN MFMAs on the fragments in `rc` from zero, each folded into the
-    // accumulators two MFMAs later with the scale of block `blk`; between them the fragment reads of the
-    // following K step into `rn` and the conversion of the next row's codes.
-    auto codes = [&](uint2_t raw) {
-        half2_t q[4];
-        nt_cvt_i8x4(raw[0], q[0], q[1]);
-        nt_cvt_i8x4(raw[1], q[2], q[3]);
-        return half8_t{q[0][0], q[0][1], q[1][0], q[1][1], q[2][0], q[2][1], q[3][0], q[3][1]};
-    };
-    half8_t Qn = codes(r0.a[0]);
-    float accs[TM][TN][4]; // the accumulators as scalars: each is written by a vector instruction of its own
-#pragma unroll
-    for (int a = 0; a < TM; a++)
-#pragma unroll
-        for (int b = 0; b < TN; b++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) accs[a][b][r] = 0.f;
-    auto k_step = [&](const Raw &rc, Raw &rn, int blk, int rstage, int rkk) {
-        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-        float4_t P[3]; // partial sums of three tiles in flight: a tile is folded two MFMAs after its own
-        half8_t Q[2];
-        Q[0] = Qn;
-        int slot = 0;
-#pragma unroll
-        for (int idx = 0; idx < TM * TN + 2; idx++) {
-            const int a = idx / TN, b = idx % TN;
-            if (idx < TM * TN) {
-                P[idx % 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(rc.b[b], Q[a & 1], zero, 0, 0, 0);
-                asm volatile("" : "+v"(P[idx % 3])); // instruction selection lets results nobody orders float: this MFMA is issued here
-                if (slot < NREAD) read_one(rstage, rkk, rn, slot++); // the fragments of the following K step
-                if (b == 0 && a + 1 < TM) Q[(a + 1) & 1] = codes(rc.a[a + 1]);
-                if (idx == TM * TN - 1) Qn = codes(rn.a[0]); // row 0 of the following K step (read by slot 0)
-            }
-            if (idx >= 2) {
-                const int fa = (idx - 2) / TN, fb = (idx - 2) % TN;
-                const float d = (float)scale_of(fa, blk);
-#pragma unroll
-                for (int r = 0; r < 4; r++) accs[fa][fb][r] = fmaf(d, P[(idx - 2) % 3][r], accs[fa][fb][r]);
-                // ... and the sums are folded here, not gathered at the end of the loop body with every partial sum kept alive
-                asm volatile("" : "+v"(accs[fa][fb][0]), "+v"(accs[fa][fb][1]), "+v"(accs[fa][fb][2]), "+v"(accs[fa][fb][3]));
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    for (int64_t kg = 0; kg < nk; kg += 4) {
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            if (u == 0) {
-                // scales of the next group of four tiles, a group ahead of their use
-                const int64_t gn = min(kg + 4, nk - 4) >> 2;
-#pragma unroll
-                for (int a = 0; a < TM; a++) sc_nxt[a] = *(const uint4_t *)(sp[a] + 8 * gn);
-            }
-            k_step(r0, r1, 2 * u, cur, 1);
-            next_tile();
-            k_step(r1, r0, 2 * u + 1, nxt, 0);
-            cur = nxt;
-            nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
-        }
-#pragma unroll
-        for (int a = 0; a < TM; a++) sc_cur[a] = sc_nxt[a];
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): no load may land in LDS after the epilogue starts reusing it
-    __syncthreads();
-    float4_t acc[TM][TN];
-#pragma unroll
-    for (int a = 0; a < TM; a++)
-#pragma unroll
-        for (int b = 0; b < TN; b++) acc[a][b] = float4_t{accs[a][b][0], accs[a][b][1], accs[a][b][2], accs[a][b][3]};
-    nt_epilogue<TM, TN, WM, WN>(g, acc, smem, s, i0, j0, wi, wj, wave, lane);
-}
-
-// ---------------------------------------------------------------------------
-// Q8_0H x f16 with the widening done by the loading wavefronts.  In gemm_nt_q8dl_kernel the four
-// multiplying wavefronts also turn every code fragment they read into f16 (50 of their 153 vector
-// instructions per K step) while the loading wavefronts' vector units idle.  Here LW = 4 loading
-// wavefronts, one per SIMD, fetch the int8 tile into registers (a lane: 16 codes of one row), widen it
-// (exact) and store f16 code tiles into the ring in the f16 kernel's swizzled layout; the activation tile still
-// goes global -> LDS directly.  The multiplying wavefronts then run the f16 kernel's fragment reads and,
-// per block of 32, one MFMA from zero whose four sums per lane are folded into the accumulators with the
-// block's f16 scale two MFMAs later, as before: no weight is rounded.
+// Q8_0H x f16.  Four loading wavefronts, one per SIMD, fetch the int8 tile into registers (a lane: 16 codes of
+// one row), widen it to f16 (exact) and store f16 code tiles into the ring in the f16 kernel's swizzled layout;
+// the activation tile goes global -> LDS directly.  The four multiplying wavefronts run the f16 kernel's
+// fragment reads and, per block of 32, one MFMA from zero whose four sums per lane are folded into the
+// accumulators with the block's f16 scale two MFMAs later (v_fma_mix: the f16 scale is an operand as it is).
+// No weight is rounded.  Two earlier forms: the operand q * d itself, exactly, as the sum of two f16
+// (hi = rn(q * d), lo = fma(q, d, -hi)) with two MFMAs per tile into the running accumulator, 64.5 us at
+// [512 x 2560] . [10240 x 2560]^T; int8 tiles in LDS, widened by the multiplying wavefronts when they read their
+// fragments (50 of their 153 vector instructions per K step), 43.2 us; this one 41.6: what is left is the
+// fold, four fused multiply-adds per MFMA, which the multiplying wavefronts cannot hand to anyone.
+// Rounding q * d to f16 (the reference's own shader does, ops/gemm.rs:547-548) would remove the fold, and was
+// measured: the outputs near zero then miss the 2e-2 tolerance (0.115).
 //
 // Ring of four stages of (BM + BN) x 64 halves.  Loading wavefront, iteration j: request the codes of tile
 // j + 3 (registers, set (j + 3) % 4) and its activation rows (LDS-DMA into stage (j + 3) % 4, last read
@@ -816,8 +610,12 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_q8w_kernel(GemmN
                                         __builtin_bit_cast(uint32_t, h[2]), __builtin_bit_cast(uint32_t, h[3])};
                     const uint4_t hi = {__builtin_bit_cast(uint32_t, h[4]), __builtin_bit_cast(uint32_t, h[5]),
                                         __builtin_bit_cast(uint32_t, h[6]), __builtin_bit_cast(uint32_t, h[7])};
-                    *(uint4_t *)(st + nt_slot(adst[c], 2 * piece)) = lo;
-                    *(uint4_t *)(st + nt_slot(adst[c], 2 * piece + 1)) = hi;
+                    // the four lanes of a row store four of its eight slots, and two neighbouring rows have the same
+                    // swizzle: odd rows store their odd slots first, so that eight consecutive lanes cover eight
+                    // different 16-byte bank groups
+                    const int flip = adst[c] & 1;
+                    *(uint4_t *)(st + nt_slot(adst[c], 2 * piece + flip)) = flip ? hi : lo;
+                    *(uint4_t *)(st + nt_slot(adst[c], 2 * piece + 1 - flip)) = flip ? lo : hi;
                 }
             }
         };
@@ -988,16 +786,6 @@ static hipError_t launch_splitk_reduce(const GemmNtArgs &g, int64_t stacks, hipS
     return hipGetLastError();
 }
 
-template <int BM, int BN, int STAGES, int LW>
-static hipError_t launch_nt_q8dl(const GemmNtArgs &g, int64_t stacks, hipStream_t st) {
-    const size_t lds = (size_t)STAGES * (BM * NT_BK + BN * NT_LDK * 2);
-    if (const hipError_t e = ensure_lds_limit<&gemm_nt_q8dl_kernel<BM, BN, STAGES, LW>>(); e != hipSuccess) return e;
-    dim3 grid((unsigned)((int64_t)g.tiles_i * g.tiles_j), (unsigned)stacks, (unsigned)g.ksplit);
-    hipLaunchKernelGGL((gemm_nt_q8dl_kernel<BM, BN, STAGES, LW>), grid, dim3(NT_THREADS + 64 * LW), lds, st, g);
-    if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-    return g.ksplit > 1 ? launch_splitk_reduce(g, stacks, st) : hipSuccess;
-}
-
 template <int BM, int BN, int LW>
 static hipError_t launch_nt_q8w(const GemmNtArgs &g, int64_t stacks, hipStream_t st) {
     const size_t lds = (size_t)4 * (BM + BN) * NT_LDK * 2;
@@ -1138,8 +926,6 @@ static hipError_t launch_nt(const GemmNtArgs &g, int64_t stacks, hipStream_t st)
 
 // Tunable: 0 = automatic, 1 = never take this kernel (for comparisons).
 RT_TUNABLE(g_gemm_nt_disable, 0);
-// Tunable: 1 = Q8_0H tiles widened by the multiplying wavefronts (gemm_nt_q8dl_kernel) instead of the loading ones.
-RT_TUNABLE(g_gemm_nt_q8_variant, 0);
 
 // f16 or Q8_0H A with K-contiguous rows, f16 B with K-contiguous rows.
 // hipErrorNotSupported: the problem does not fit; the generic tiled GEMM runs instead.
@@ -1253,7 +1039,7 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
                                      : launch_nt_dl<BM, BN, 3, 2>(g, p.stacks, stream);
     }
     if (dl_q8)
-        return g_gemm_nt_q8_variant == 1 ? launch_nt_q8dl<BM, BN, 4, 2>(g, p.stacks, stream) : launch_nt_q8w<BM, BN, 4>(g, p.stacks, stream);
+        return launch_nt_q8w<BM, BN, 4>(g, p.stacks, stream);
     if (q8) return kfull ? launch_nt<BM, BN, true, true>(g, p.stacks, stream) : launch_nt<BM, BN, true, false>(g, p.stacks, stream);
     return kfull ? launch_nt<BM, BN, false, true>(g, p.stacks, stream) : launch_nt<BM, BN, false, false>(g, p.stacks, stream);
 }
