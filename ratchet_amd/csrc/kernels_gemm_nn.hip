@@ -2,25 +2,28 @@
 // (+ bias), A rows K-contiguous, B rows N-contiguous, N <= 128, C row-major.  This is the
 // attention P.V form (P [seq x seq], V [seq x head_dim]): a stream over A, read exactly once.
 //
-// A workgroup of eight wavefronts owns 64 rows of A and all of N.  A is used once, so it never
-// touches LDS: lane (fr, fg) loads the 16 bytes A[row fr][32 kh + 8 fg ..] that are its operand
-// of a K step.  B is shared by the workgroup and goes through LDS as it lies in memory, [k][n]:
-// ds_read_b64_tr_b16 hands each lane the four consecutive k of one column that an MFMA operand
-// wants (within 16 lanes, lane s addresses columns 4 (s % 4) .. + 3 of row s / 4 and lane i
-// receives column i of the four rows), so nothing is transposed by hand.  Per K tile of 64 the
-// wavefronts 0..3 multiply their 16 rows by the tile's first 32 rows of B and the wavefronts 4..7
-// by the other 32 (v_mfma_f32_16x16x32_f16); the two partial sums meet in LDS at the end.  Two LDS
-// stages, one barrier per tile; the loads of the next seven tiles are in flight in registers: at
-// the sizes this kernel sees (a few tens of MB) the whole problem has to be requested at once to
-// keep HBM busy.  The result is staged in LDS and written with 128-bit stores.
+// A workgroup of eight wavefronts owns 64 rows of A and all of N.  A is used once and read in whole
+// lines: wavefronts 0..3 take the even K tiles of 64 and 4..7 the odd ones, a wavefront's two loads
+// per tile are its 16 rows x 128 bytes (eight lanes per row), which it passes through a 2 KiB LDS region
+// of its own (swizzled rows; LDS operations of one wavefront complete in order, no barrier) to come
+// back as the MFMA operands of the tile's two K steps.  B is shared by the workgroup and goes through
+// LDS as it lies in memory, [k][n]: ds_read_b64_tr_b16 hands each lane the four consecutive k of one
+// column that an MFMA operand wants (within 16 lanes, lane s addresses columns 4 (s % 4) .. + 3 of row
+// s / 4 and lane i receives column i of the four rows), so nothing is transposed by hand.  B tiles go
+// to LDS in pairs (four stages, one barrier per pair); four pairs are in flight in registers: at the sizes
+// this kernel sees (a few tens of MB) the whole problem has to be requested at once to keep HBM busy.
+// The two wavefront groups' partial sums meet in LDS at the end; the result is staged in LDS and written
+// with 128-bit stores.
 //
 // EXACT: M and K are multiples of 64, N of 16 and a workgroup's operands span less than 2 GiB: no
 // clamps or zero fills, and every load is a wave-uniform base plus a 32-bit lane offset fixed for
 // the whole kernel.
 //
-// Measured on the attention shape (32 x [512 x 512] . [512 x 80], 22 MB): loads alone 8.5 us, of
-// which A alone 7.6 (6.8 if a wavefront read whole rows instead of 16 rows x 64 bytes), LDS stores
-// and barriers + 0.3, transposing reads and MFMAs + 1.4; the arithmetic alone, without the loads, 4.1.
+// Measured on the attention shape (32 x [512 x 512] . [512 x 80], 22 MB): 9.6 us.  The form before
+// loaded A straight into MFMA operand layout, 16 rows x 64 bytes per instruction (half a line per row):
+// 10.2 us; a read-only probe over the 16.8 MB of A takes 5.2 us in that pattern and 3.9 us in this one.
+// Of the rest, the arithmetic alone (LDS stores and barriers, transposing reads, MFMAs, epilogue), without
+// the loads, takes 4.1 us.
 //
 // Role in the reference: ops/gemm.rs:305-657 with trans_rhs = false (phi2 / whisper attention,
 // `matmul(V, false, false)`).
@@ -41,179 +44,10 @@ struct GemmNnArgs {
 
 constexpr int NN_BK = 64;
 
-constexpr int NNT_BM = 64, NNT_DEPTH = 8, NNT_THREADS = 512;
+constexpr int NNT_BM = 64, NNT_THREADS = 512;
 
 template <int TN, bool EXACT>
 __global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr_kernel(GemmNnArgs g) {
-    constexpr int NP = 16 * TN;                        // padded N
-    constexpr int BR = NP + 8;                         // halfs per row of the B tile
-    constexpr int B_VECS = NN_BK * (NP / 8);           // 16-byte vectors of a full B tile
-    constexpr int B_VEC = (B_VECS + NNT_THREADS - 1) / NNT_THREADS; // per thread
-    constexpr int STAGE = NN_BK * BR;
-    constexpr int EROW = NP + 8;
-    constexpr int RED_FLOATS = 4 * TN * 4 * 64;        // the second wavefront group's accumulators
-    static_assert(NN_BK == 64, "two K steps per tile, one per wavefront group");
-
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    half_t *S0 = (half_t *)smem; // [2][64][BR]; afterwards the partial sums [4][TN][4][64] f32 and the output staging
-
-    const int t = threadIdx.x, lane = t & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int rw = wave & 3, kh = wave >> 2; // 16 rows of A, and which K step of every tile
-    const int fr = lane & 15, fg = lane >> 4;
-    // Workgroups go to the eight XCDs round robin by their linear index, and each XCD has its own L2:
-    // the row blocks of one stack share its B, so they are given indices that land on one XCD.
-    const uint32_t mb = (uint32_t)((g.M + NNT_BM - 1) / NNT_BM), nstacks = gridDim.x / mb;
-    uint32_t blk = blockIdx.x % mb, stk = blockIdx.x / mb;
-    if (nstacks % 8 == 0) {
-        const uint32_t idx = blockIdx.x >> 3;
-        stk = (blockIdx.x & 7) + 8 * (idx / mb), blk = idx % mb;
-    }
-    const int64_t i0 = (int64_t)blk * NNT_BM;
-    const int64_t s = stk;
-    const half_t *A = g.A + (g.a_stack == 1 ? 0 : s) * g.a_bs;
-    const half_t *B = g.B + (g.b_stack == 1 ? 0 : s) * g.b_bs;
-    const int nvec = EXACT ? NP / 8 : (int)(g.N >> 3);
-    const uint4_t zero4 = {0u, 0u, 0u, 0u};
-
-    // this lane's row of A (rows past the end duplicate the last one), its K offset inside a tile, and
-    // its vectors of the B tile: vector v = t + 512 i is (row v / nvec, column 8 (v % nvec))
-    const int arow = rw * 16 + fr, ak = 32 * kh + 8 * fg;
-    const half_t *ap = A + min(i0 + arow, g.M - 1) * g.a_rs + ak;
-    int bk[B_VEC], bc[B_VEC];
-#pragma unroll
-    for (int i = 0; i < B_VEC; i++) {
-        const int v = min(t + NNT_THREADS * i, NN_BK * nvec - 1);
-        bk[i] = v / nvec, bc[i] = v - bk[i] * nvec;
-    }
-    // EXACT: byte offsets from the tile's first byte
-    const uint32_t aoff = 2u * (uint32_t)(arow * (int)g.a_rs + ak);
-    uint32_t boff[B_VEC];
-#pragma unroll
-    for (int i = 0; i < B_VEC; i++) boff[i] = 2u * (uint32_t)(bk[i] * (int)g.b_ks + 8 * bc[i]);
-    const char *abase = (const char *)(A + i0 * g.a_rs);
-    const int64_t b_tile_bytes = 2 * NN_BK * g.b_ks;
-    auto b_mine = [&](int i) { return NNT_THREADS * (i + 1) <= B_VECS || t + NNT_THREADS * i < (EXACT ? B_VECS : NN_BK * nvec); };
-
-    constexpr int D = NNT_DEPTH;
-    uint4_t ra_[D], rb_[D][B_VEC];
-    auto load_tiles = [&](int64_t k0, uint4_t &ra, uint4_t (&rb)[B_VEC]) {
-        if constexpr (EXACT) {
-            const char *at = abase + 2 * k0, *bt = (const char *)B + (k0 / NN_BK) * b_tile_bytes; // uniform
-#pragma unroll
-            for (int i = 0; i < B_VEC; i++) rb[i] = *(const uint4_t *)(bt + boff[i]); // (threads without a vector re-read the last one)
-            ra = *(const uint4_t *)(at + aoff);
-        } else {
-#pragma unroll
-            for (int i = 0; i < B_VEC; i++) rb[i] = *(const uint4_t *)(B + min(k0 + bk[i], g.K - 1) * g.b_ks + 8 * bc[i]);
-            const uint4_t v = *(const uint4_t *)(ap + min(k0, g.K - 8 - ak)); // past K: a valid vector, replaced by zeros
-            ra = k0 + ak < g.K ? v : zero4;
-        }
-    };
-    // registers -> LDS: B rows as they are (rows past K zeroed: the padded part of the last K tile adds nothing)
-    auto store_tile = [&](half_t *st, int64_t k0, const uint4_t (&rb)[B_VEC]) {
-        const bool full = EXACT || k0 + NN_BK <= g.K; // uniform: only the last tile can be ragged
-#pragma unroll
-        for (int i = 0; i < B_VEC; i++)
-            if (b_mine(i)) *(uint4_t *)(st + bk[i] * BR + 8 * bc[i]) = (full || k0 + bk[i] < g.K) ? rb[i] : zero4;
-    };
-
-    float4_t acc[TN];
-#pragma unroll
-    for (int b = 0; b < TN; b++) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
-    // byte address in LDS of the first row / columns this lane addresses for B
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const half_t *)S0;
-    const uint32_t b_off = lds0 + 2u * (uint32_t)((32 * kh + 8 * fg + (fr >> 2)) * BR + 4 * (fr & 3));
-
-    const int nk = (int)((g.K + NN_BK - 1) / NN_BK);
-    auto tile_k0 = [&](int kt) { return (int64_t)kt * NN_BK; };
-    // (unconditional: a branch here would leave the compiler unable to count the loads in flight, and it
-    // would then wait for all of them before the first tile; short problems load their last tile again)
-#pragma unroll
-    for (int d = 0; d < D - 1; d++) {
-        load_tiles(tile_k0(min(d, nk - 1)), ra_[d], rb_[d]);
-        __builtin_amdgcn_sched_barrier(0); // in this order: the first tile's data is waited for first
-    }
-    auto trip = [&](int kt0) {
-#pragma unroll
-        for (int u = 0; u < D; u++) {
-            const int kt = kt0 + u;
-            if (kt < nk) { // uniform
-                if (kt + D - 1 < nk) load_tiles(tile_k0(kt + D - 1), ra_[(u + D - 1) % D], rb_[(u + D - 1) % D]);
-                store_tile(S0 + (u & 1) * STAGE, tile_k0(kt), rb_[u]); // D is even: tile kt lives in stage kt % 2
-                // everybody's stores of this tile are done; everybody has finished with the other stage's last tile
-                __syncthreads();
-                const uint32_t sb = b_off + 2u * (uint32_t)((u & 1) * STAGE);
-                uint64_t lo[TN], hi[TN];
-#pragma unroll
-                for (int b = 0; b < TN; b++)
-                    asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
-                                 : "=&v"(lo[b]), "=&v"(hi[b])
-                                 : "v"(sb), "n"(2 * 16 * b), "n"(2 * (16 * b + 4 * BR))
-                                 : "memory");
-#pragma unroll
-                for (int b = 0; b < TN; b++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[b]), "+v"(hi[b])::"memory");
-                typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
-                const half8_t fa = __builtin_bit_cast(half8_t, ra_[u]);
-#pragma unroll
-                for (int b = 0; b < TN; b++)
-                    acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, __builtin_bit_cast(half8_t, u64x2_t{lo[b], hi[b]}), acc[b], 0, 0, 0);
-            }
-        }
-    };
-    // The first D tiles stand outside the loop: at a loop header the compiler's count of loads in flight
-    // is the cautious merge of both ways in, and it would wait for all of them before the first tile.
-    trip(0);
-    for (int kt0 = D; kt0 < nk; kt0 += D) trip(kt0);
-    __syncthreads(); // the stages become the partial sums and the output staging
-
-    // the second group hands its sums to the first
-    float4_t *red = (float4_t *)smem + rw * TN * 64;
-    if (kh == 1) {
-#pragma unroll
-        for (int b = 0; b < TN; b++) red[b * 64 + lane] = acc[b];
-    }
-    __syncthreads();
-    if (kh == 1) return;
-#pragma unroll
-    for (int b = 0; b < TN; b++) acc[b] += red[b * 64 + lane];
-
-    // acc[b][r] is row 4 * fg + r of the wavefront's 16, column 16 * b + fr
-    half_t *es = (half_t *)(smem + 4 * RED_FLOATS) + rw * 16 * EROW;
-    rt_with_act(g.act, [&](auto has_act) {
-#pragma unroll
-        for (int b = 0; b < TN; b++) {
-            const int n = 16 * b + fr;
-            float bn = 0.f;
-            if (g.has_bias && !g.bias_on_rows) bn = (float)g.bias[min(n, (int)g.N - 1)];
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int il = 4 * fg + r;
-                float v = acc[b][r] + bn;
-                if (g.has_bias && g.bias_on_rows) v += (float)g.bias[min(i0 + rw * 16 + il, g.M - 1)];
-                v = rt_act_k<decltype(has_act)::value>(v);
-                es[il * EROW + n] = (half_t)v;
-            }
-        }
-    });
-    asm volatile("" ::: "memory"); // read back by the same wavefront; DS operations complete in order
-    half_t *out = g.out + s * g.o_bs;
-    for (int v = lane; v < 16 * nvec; v += 64) {
-        const int il = v / nvec, c = v - il * nvec;
-        const int64_t i = i0 + rw * 16 + il;
-        if (i < g.M) __builtin_nontemporal_store(*(const uint4_t *)(es + il * EROW + 8 * c), (uint4_t *)(out + i * g.o_is + 8 * c));
-    }
-}
-
-// The same product with A read in whole lines.  In gemm_nn_tr_kernel a load instruction fetches 16 rows x 64
-// bytes, half a line per row; a read-only probe over the 16.8 MB of the attention shape's A takes 5.2 us in that
-// pattern and 3.9 us when eight lanes share a row and a load fetches 8 rows x 128 bytes.  Here wavefronts
-// 0..3 take the even K tiles and 4..7 the odd ones, whole tiles: a wavefront's two loads per tile are its 16 rows
-// x 128 bytes, which it passes through a 2 KiB LDS region of its own (swizzled rows; LDS operations of one
-// wavefront complete in order, no barrier) to come back as the MFMA operands of the tile's two K steps.  B tiles
-// go to LDS in pairs, four stages, one barrier per pair; four pairs are in flight in registers.
-template <int TN, bool EXACT>
-__global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr2_kernel(GemmNnArgs g) {
     constexpr int NP = 16 * TN;
     constexpr int BR = NP + 8;
     constexpr int B_VECS = NN_BK * (NP / 8);
@@ -282,7 +116,7 @@ __global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr2_kernel(GemmNnArgs g) 
             const char *at = abase + 2 * k0;
             ra[0] = *(const uint4_t *)(at + aoff0), ra[1] = *(const uint4_t *)(at + aoff1);
         } else {
-            const int64_t kc = min(k0, g.K - 8 - 8 * ap); // K >= 64 here (the launcher sees to it)
+            const int64_t kc = max(min(k0, g.K - 8 - 8 * ap), (int64_t)(-8 * ap)); // the vector read lies inside the row whatever K is
             const uint4_t v0 = *(const uint4_t *)(ap0 + kc), v1 = *(const uint4_t *)(ap1 + kc);
             const bool in = k0 + 8 * ap < g.K;
             ra[0] = in ? v0 : zero4, ra[1] = in ? v1 : zero4;
@@ -311,23 +145,29 @@ __global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr2_kernel(GemmNnArgs g) 
         *(uint4_t *)(T + tslot(ar + 8, ap)) = ra[1];
         asm volatile("" ::: "memory");
         const uint32_t sb = b_off + 2u * (uint32_t)((2 * (q & 1) + grp) * STAGE);
+        // both K steps' operands are requested before the first MFMA: one trip through the LDS latency per tile
+        half8_t fa[2];
+        uint64_t lo[2][TN], hi[2][TN];
 #pragma unroll
         for (int ks = 0; ks < 2; ks++) {
-            const half8_t fa = __builtin_bit_cast(half8_t, *(const uint4_t *)(T + tslot(fr, 4 * ks + fg)));
-            uint64_t lo[TN], hi[TN];
+            fa[ks] = __builtin_bit_cast(half8_t, *(const uint4_t *)(T + tslot(fr, 4 * ks + fg)));
 #pragma unroll
             for (int b = 0; b < TN; b++)
                 asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
-                             : "=&v"(lo[b]), "=&v"(hi[b])
+                             : "=&v"(lo[ks][b]), "=&v"(hi[ks][b])
                              : "v"(sb + 2u * (uint32_t)(32 * ks * BR)), "n"(2 * 16 * b), "n"(2 * (16 * b + 4 * BR))
                              : "memory");
+        }
 #pragma unroll
-            for (int b = 0; b < TN; b++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[b]), "+v"(hi[b])::"memory");
-            typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int b = 0; b < TN; b++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[ks][b]), "+v"(hi[ks][b])::"memory");
+        typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
 #pragma unroll
             for (int b = 0; b < TN; b++)
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, __builtin_bit_cast(half8_t, u64x2_t{lo[b], hi[b]}), acc[b], 0, 0, 0);
-        }
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[ks], __builtin_bit_cast(half8_t, u64x2_t{lo[ks][b], hi[ks][b]}), acc[b], 0, 0, 0);
     };
     // (unconditional: a branch here would leave the compiler unable to count the loads in flight)
 #pragma unroll
@@ -388,23 +228,14 @@ __global__ __launch_bounds__(NNT_THREADS) void gemm_nn_tr2_kernel(GemmNnArgs g) 
     }
 }
 
-// Tunable: 1 = the kernel whose loads fetch 16 rows x 64 bytes (for comparisons).
-RT_TUNABLE(g_gemm_nn_halflines, 0);
-
 template <int TN> static hipError_t launch_nn_tr(const GemmNnArgs &g, int64_t stacks, hipStream_t st) {
     constexpr int NP = 16 * TN;
-    const size_t lds = std::max<size_t>((size_t)2 * NN_BK * (NP + 8) * 2, (size_t)4 * 4 * TN * 4 * 64 + (size_t)4 * 16 * (NP + 8) * 2);
+    const size_t lds = std::max<size_t>((size_t)4 * NN_BK * (NP + 8) * 2 + 8 * 16 * 64 * 2, (size_t)4 * 4 * TN * 4 * 64 + (size_t)4 * 16 * (NP + 8) * 2);
     dim3 grid((unsigned)((g.M + NNT_BM - 1) / NNT_BM * stacks));
     const bool exact = g.M % NNT_BM == 0 && g.K % NN_BK == 0 && g.N == NP && g.a_rs < (1 << 23) && g.K * g.b_ks < (1 << 29);
-    if (!g_gemm_nn_halflines && g.K >= NN_BK) {
-        const size_t lds2 = std::max<size_t>((size_t)4 * NN_BK * (NP + 8) * 2 + 8 * 16 * 64 * 2, (size_t)4 * 4 * TN * 4 * 64 + (size_t)4 * 16 * (NP + 8) * 2);
-        if (lds2 > 48 * 1024) {
-            const hipError_t e = exact ? ensure_lds_limit<&gemm_nn_tr2_kernel<TN, true>>() : ensure_lds_limit<&gemm_nn_tr2_kernel<TN, false>>();
-            if (e != hipSuccess) return e;
-        }
-        if (exact) hipLaunchKernelGGL((gemm_nn_tr2_kernel<TN, true>), grid, dim3(NNT_THREADS), lds2, st, g);
-        else hipLaunchKernelGGL((gemm_nn_tr2_kernel<TN, false>), grid, dim3(NNT_THREADS), lds2, st, g);
-        return hipGetLastError();
+    if (lds > 48 * 1024) {
+        const hipError_t e = exact ? ensure_lds_limit<&gemm_nn_tr_kernel<TN, true>>() : ensure_lds_limit<&gemm_nn_tr_kernel<TN, false>>();
+        if (e != hipSuccess) return e;
     }
     if (exact) hipLaunchKernelGGL((gemm_nn_tr_kernel<TN, true>), grid, dim3(NNT_THREADS), lds, st, g);
     else hipLaunchKernelGGL((gemm_nn_tr_kernel<TN, false>), grid, dim3(NNT_THREADS), lds, st, g);
