@@ -345,8 +345,6 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
             e = rt::launch_gemm_f32(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
         // Q4_K weights against many activation rows
         if (e == hipErrorNotSupported)
-            e = rt::launch_gemm_q4k_reg(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-        if (e == hipErrorNotSupported)
             e = rt::launch_gemm_q4k(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
         if (e == hipErrorNotSupported)
             e = rt::launch_gemm(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);

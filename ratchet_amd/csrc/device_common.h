@@ -158,8 +158,6 @@ hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, 
                                 hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
                                const DeviceInfo &dev);
-hipError_t launch_gemm_q4k_reg(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
-                               const DeviceInfo &dev);
 hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
                            const DeviceInfo &dev);
 hipError_t launch_gemm_f32(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,

@@ -1,24 +1,40 @@
-// Q4_K weights x f16 activations for many activation rows (prefill): a tiled GEMM whose K tile is
-// half a super-block (128), with one scale application per super-block.
+// Q4_K weights x f16 activations for many activation rows (prefill), the weights never touching LDS:
+// every multiplying wavefront decodes the raw blocks of its own 32 weight rows in registers, straight
+// into the MFMA operand, and only the activation tile goes through LDS.
 //
 //   y[j, i] = sum_sb ( d_i,sb * sum_sub sum_{k in sub} x[j,k] (sc_i,sub q_i,k)  -  dmin_i,sb * sum_sub mn_i,sub S[j,sub] )
 //   S[j, sub] = sum_{k in sub} x[j, k]
 //
-// The same exact-operand scheme as the streaming kernel (kernels_gemv_q4k_mfma.hip): sc * q < 1024
-// is exact in f16, so the eight sub-blocks of a super-block chain through one MFMA accumulator and
-// d is applied once per super-block in f32; the sub-block sums of x come out of an MFMA against
-// ones, are split into f16 high + low parts (exact to 2^-22) and meet the integer mins in one more
-// MFMA pair.  No weight is rounded.
+// The order of K inside an MFMA is free as long as both operands agree, so lane group g (lane / 16)
+// of a weight fragment owns the 32 bytes g of a super-block's qs: the low nibbles are the values
+// 64 g .. + 31 of the super-block (sub-block 2 g), the high nibbles the values 64 g + 32 .. + 63
+// (sub-block 2 g + 1).  MFMA step t of a super-block takes from lane group g the values
+// 64 g + 8 t .. + 7: bytes 8 (t % 4) .. + 7, low nibbles for t < 4, high for t >= 4.  A thread
+// therefore reads a header and two 16-byte pieces per super-block and needs two of the eight scales
+// and mins.  sc * q < 1024 is exact in f16 (fma(1024 + q, sc, -1024 sc) rounds once; the high
+// nibbles stay in place as 1024 + 16 q against sc / 16), so a super-block chains through one MFMA
+// accumulator and d is applied once per super-block in f32.  No weight is rounded.
 //
-// A workgroup owns 64 weight rows x 128 activation rows and steps K by half a super-block.  Eight
-// wavefronts multiply (2 x 4, 32 weight rows x 32 activation rows each: 16 + 8 MFMAs per tile and
-// 8 more per super-block for the min term); each of their threads turns 8 bytes of qs into 16 values
-// of sc * q per tile, in registers between the MFMAs of the tile before, and stores them into the
-// other of two LDS stages.  A ninth wavefront only issues LDS-DMA loads of the activation tiles, two
-// tiles ahead in a ring of three stages, so the multiplying wavefronts hold no activations in
-// registers and wait for nothing but their own small loads of raw blocks.  One barrier per tile.
-// The generic kernel's K tile is one sub-block of 32: a store / barrier / read / MFMA / fold /
-// barrier chain per 32 values of K that nothing overlapped.
+// The sub-block sums of x fall out of the same layout: a lane of an activation fragment holds
+// 8 values of sub-block 2 g (t < 4) or 2 g + 1 (t >= 4) of activation row lane % 16, so four dot
+// products against ones per step give S for exactly the (row, sub-block pair) that the min-term MFMA
+// wants from this lane.  Wavefront w sums the 16 activation rows of fragment w and shares them
+// through LDS (f16 high + low parts, exact to 2^-22); the min term of super-block sb is one MFMA per
+// output tile, run under super-block sb + 1.
+//
+// A workgroup owns 128 weight rows x 64 activation rows: four multiplying wavefronts (32 weight rows
+// x 64 activation rows each: 64 MFMAs per super-block, 8 for the min term) and four that only issue
+// the activation tiles' LDS-DMA loads (one per SIMD, so that no multiplying wavefront shares its SIMD
+// with all of them), two super-blocks ahead in a ring of three stages.  A staged row is 32 K-vectors
+// and one of padding: the 16 rows of a fragment read start 4 banks apart and a read address is a
+// base + 16 * step, an immediate.  One barrier per super-block.  The output tile leaves through LDS
+// as 16-byte stores when the output is contiguous along the weight rows.
+//
+// What bounds it (measured by leaving parts out): the parts add up.  A wavefront's MFMAs (8 issue
+// cycles each when vector instructions follow), its 335 vector instructions per super-block and the
+// LDS pipe time of the compute unit's fragment reads (128 KB per super-block at 128 B/clk) each
+// cost their full time whatever the order of instructions; two multiplying wavefronts per SIMD would
+// need the decoding done twice or more registers than a SIMD has.
 //
 // The arithmetic is ggml's dequantize_row_q4_K (the reference holds only the block struct,
 // crates/ratchet-loader/src/k_quants.rs:94-103); the caller convention is Linear's
@@ -32,99 +48,65 @@ struct GemmQ4kArgs {
     const half_t *X;
     const half_t *bias;
     half_t *out;
-    int64_t M, N, K; // weight rows, activation rows, contraction
-    int64_t nsb;     // super-blocks per row
+    int64_t M, N; // weight rows, activation rows
+    int64_t nsb;  // super-blocks per row
     int64_t a_stack, b_stack;
     int64_t b_bs, b_js;
     int64_t o_bs, o_is, o_js;
-    int tiles_j;
+    int tiles_j, remap, vec_out;
     int has_bias, bias_on_rows, act;
 };
 
-constexpr int QK_BM = 64, QK_BN = 128; // weight rows x activation rows per workgroup
-constexpr int QK_KT = 128;             // K per tile: half a super-block, so that several LDS stages fit
-constexpr int QK_WLD = QK_KT + 8;      // halfs per weight row in LDS: the 16 rows of a fragment read start 16 bytes apart in the banks
-constexpr int QK_XS = QK_BN * QK_KT;   // halfs per activation stage: rows unpadded (LDS-DMA writes 1 KB runs), 16-byte slots XOR-swizzled
-constexpr int QK_WS = QK_BM * QK_WLD;  // halfs per weight stage
-constexpr int QK_LW = 1;               // wavefronts that only issue the activation tiles' LDS-DMA
-constexpr int QK_THREADS = 512 + 64 * QK_LW; // eight multiplying wavefronts, two per SIMD: one's MFMAs run under the other's decoding
-constexpr int QK_XST = 3;              // activation stages: a tile's slots are in flight for two tiles
-constexpr size_t QK_LDS = (size_t)(QK_XST * QK_XS + 2 * QK_WS) * 2 + QK_BM * 8 * 2 + 2 * QK_BM * 4;
+constexpr int QR_BM = 128, QR_BN = 64; // weight rows x activation rows per workgroup
+// An activation stage holds one super-block of K for 64 rows: 32 K-vectors of 16 bytes per row and one of padding,
+// so that the 16 rows of a fragment read start 4 banks apart and a read address is base + 16 * step.
+constexpr int QR_ROWB = 33 * 16;       // bytes per staged row
+constexpr int QR_XSB = QR_BN * QR_ROWB; // bytes per stage = 33 LDS-DMA instructions of 1 KB
+constexpr int QR_XST = 3;              // activation stages: a tile's slots are in flight for two super-blocks
+constexpr int QR_LW = 4;               // wavefronts that only issue the LDS-DMA, one per SIMD
+constexpr int QR_THREADS = 256 + 64 * QR_LW;
+constexpr size_t QR_LDS = (size_t)QR_XST * QR_XSB + 2 * QR_BN * 4 * 8;
 
-// 4 bytes holding integers 0..255 -> two half2 holding 1024 + the same integers
-__device__ __forceinline__ void qk_bytes_to_biased(uint32_t v, half2_t &lo, half2_t &hi) {
-    lo = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u));
-    hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u));
-}
-
-// 8 nibble-bytes (two dwords, each byte 0..15) times sc -> 8 halfs, exactly:
-// fma(1024 + q, sc, -1024 sc) rounds once and q * sc < 1024 is representable.
-__device__ __forceinline__ uint4_t qk_scaled8(uint32_t v0, uint32_t v1, half_t sc) {
-    const half2_t s2 = {sc, sc};
-    const half_t n = (half_t)(-1024.0f * (float)sc);
-    const half2_t n2 = {n, n};
-    half2_t a, b, c, d;
-    qk_bytes_to_biased(v0, a, b);
-    qk_bytes_to_biased(v1, c, d);
-    a = __builtin_elementwise_fma(a, s2, n2), b = __builtin_elementwise_fma(b, s2, n2);
-    c = __builtin_elementwise_fma(c, s2, n2), d = __builtin_elementwise_fma(d, s2, n2);
-    return uint4_t{__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), __builtin_bit_cast(uint32_t, c),
-                   __builtin_bit_cast(uint32_t, d)};
-}
-
-__global__ __launch_bounds__(QK_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
-    constexpr int TA = 2, TB = 2; // MFMA tiles per wavefront: weight rows (second operand), activation rows (first)
+__global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
+    constexpr int TA = 2, TB = 4; // MFMA tiles per wavefront: weight rows (second operand), activation rows (first)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    half_t *Xs = (half_t *)smem;           // [QK_XST][QK_BN][QK_KT]  activations of tile kt in stage kt % 3, slot c of row r at slot c ^ (r % 16)
-    half_t *Ws = Xs + QK_XST * QK_XS;     // [2][QK_BM][QK_WLD]  sc * q of tile kt in stage kt % 2
-    half_t *Mn = Ws + 2 * QK_WS;           // [64][8]   mins of the 8 sub-blocks of the current super-block, as f16 integers
-    float *Ds = (float *)(Mn + QK_BM * 8); // [64] d, then [64] dmin
-    float *Dm = Ds + QK_BM;
+    uint8_t *Xs = smem;                             // [QR_XST][64 rows][33 slots of 16 bytes]: K-vector v of row r in slot v
+    uint2_t *Sx = (uint2_t *)(Xs + QR_XST * QR_XSB); // [2][64][4]: sums of x of super-block parity p, row, lane group: (high pair, low pair)
 
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wi = wave >> 2, wj = wave & 3; // 2 x 4 wavefronts of 32 weight rows x 32 activation rows
     const int fr = lane & 15, fg = lane >> 4;
     const int64_t s = blockIdx.y;
-    const int64_t ti = blockIdx.x / g.tiles_j, tj = blockIdx.x - ti * g.tiles_j;
-    const int64_t i0 = ti * QK_BM, j0 = tj * QK_BN;
+    // the workgroups of one weight row block (one per block of activation rows) run on one XCD, whose L2 then
+    // holds that block's raw weights for all of them
+    uint32_t b = blockIdx.x;
+    if (g.remap) b = (b & 7) * (gridDim.x >> 3) + (b >> 3);
+    const uint32_t ti = b / (uint32_t)g.tiles_j, tj = b - ti * (uint32_t)g.tiles_j;
+    const int64_t i0 = (int64_t)ti * QR_BM, j0 = (int64_t)tj * QR_BN;
     const uint8_t *blocks = g.blocks + (g.a_stack == 1 ? 0 : s) * g.M * g.nsb * 144;
     const half_t *X = g.X + (g.b_stack == 1 ? 0 : s) * g.b_bs;
-    const int64_t last = 2 * g.nsb - 1; // tiles are numbered 2 sb + h, h = the half of the super-block
+    const int64_t last = g.nsb - 1;
+    const bool vec_out = g.vec_out && i0 + QR_BM <= g.M; // a whole tile of weight rows, stored 16 bytes at a time
 
-    // ---- what a multiplying thread moves per tile: 8 bytes of qs (piece t % 8 of weight row t / 8: 16 nibbles
-    // of two sub-blocks) with that row's header.  Rows past the end repeat the last valid one.  Offsets are
-    // 32-bit from wave-uniform bases (the launcher checks the ranges).
-    const int qrow = t >> 3, qp = t & 7;
-    const uint32_t qoff = (uint32_t)min(i0 + qrow, g.M - 1) * (uint32_t)g.nsb * 144u;
-    struct Raw {
-        uint4_t hdr;
-        uint2_t q;
-    };
-    auto load_raw = [&](int64_t kt, Raw &r) {
-        const uint8_t *bsb = blocks + (kt >> 1) * 144; // wave-uniform
-        r.hdr = *(const uint4_t *)(bsb + qoff);
-        r.q = *(const uint2_t *)(bsb + (qoff + 16u + 64u * (uint32_t)(kt & 1) + 32u * (qp >> 2) + 8u * (qp & 3)));
-    };
-    if (wave >= 8) {
-        // ---- loading wavefront: instruction i fills the 1 KB run of rows 4 i .. + 3 of a stage; lane l lands in
-        // row l / 16 of them, slot l % 16, which must hold K-vector (l % 16) ^ (row % 16) of that row.  It keeps
-        // two tiles in flight and meets the others at every tile's barrier.
-        constexpr int NI = 32 / QK_LW;
-        const int lw = wave - 8;
+    if (wave >= 4) {
+        // ---- loading wavefront lw: LDS-DMA instruction i of a stage (i = lw, lw + 4, ...; 33 in all) fills the 1 KB
+        // run of slots 64 i .. + 63; slot p is K-vector p % 33 of row p / 33 (the 33rd is padding and repeats the 32nd).
+        // Each of the four issues nine: the ninth of wavefronts 1..3 repeats instruction 32.
+        constexpr int NI = 9;
+        const int lw = wave - 4;
         uint32_t xsrc[NI];
 #pragma unroll
-        for (int i = 0; i < NI; i++) {
-            const int row = (i * QK_LW + lw) * 4 + (lane >> 4);
-            xsrc[i] = (uint32_t)min(j0 + row, g.N - 1) * (uint32_t)g.b_js + 8u * ((lane & 15) ^ (row & 15));
+        for (int n = 0; n < NI; n++) {
+            const uint32_t p = 64u * (uint32_t)min(4 * n + lw, 32) + (uint32_t)lane;
+            const uint32_t row = p / 33u, v = min(p - 33u * row, 31u);
+            xsrc[n] = (uint32_t)min(j0 + (int64_t)row, g.N - 1) * (uint32_t)g.b_js + 8u * v;
         }
-        auto issue_x = [&](int stage, int64_t kt) {
-            const half_t *xk = X + kt * QK_KT;
+        auto issue_x = [&](int stage, int64_t sb) {
+            const half_t *xk = X + sb * 256;
 #pragma unroll
-            for (int i = 0; i < NI; i++)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xk + xsrc[i]),
-                                                 (__attribute__((address_space(3))) void *)(Xs + stage * QK_XS + (i * QK_LW + lw) * 512), 16,
-                                                 0, 0);
+            for (int n = 0; n < NI; n++)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xk + xsrc[n]),
+                                                 (__attribute__((address_space(3))) void *)(Xs + stage * QR_XSB + min(4 * n + lw, 32) * 1024), 16, 0, 0);
         };
         constexpr int kOlder = 0x0F70 | (NI & 0xF) | (((NI >> 4) & 0x3) << 14); // all but the newest tile have landed
         auto publish = [&]() {
@@ -134,53 +116,83 @@ __global__ __launch_bounds__(QK_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
             asm volatile("" ::: "memory");
         };
         issue_x(0, 0);
-        issue_x(1, 1);
-        publish(); // tile 0
+        issue_x(1, min((int64_t)1, last));
+        publish(); // super-block 0
         int fill = 2;
-        for (int64_t kt = 0; kt < last; kt++) {
-            // stage `fill` held tile kt - 1, read for the last time before the barrier just passed
-            issue_x(fill, min(kt + 2, last)); // past the end: the last tile again, into a stage nobody reads
-            publish();                        // tile kt + 1
-            fill = fill == QK_XST - 1 ? 0 : fill + 1;
+        for (int64_t sb = 0; sb < last; sb++) {
+            // stage `fill` held super-block sb - 1, read for the last time before the barrier just passed
+            issue_x(fill, min(sb + 2, last)); // past the end: the last one again, into a stage nobody reads
+            publish();                        // super-block sb + 1
+            fill = fill == QR_XST - 1 ? 0 : fill + 1;
         }
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): nothing lands after the wavefront has ended
+        __builtin_amdgcn_s_barrier();       // the multiplying wavefronts' last exchange of sums
+        if (vec_out) __builtin_amdgcn_s_barrier(); // and their staged output tile
         return;
     }
 
-    // Decodes this thread's piece of a tile of half H and stores it into stage H (tile 2 sb + h lives in
-    // stage h).  Piece p covers bytes 8 (p % 4) .. + 7 of chunk 2 H + p / 4: the low nibbles are values
-    // 8 (p % 4) .. + 7 of sub-block 2 (p / 4) of this half, the high nibbles the same values of the next one.
-    auto decode_store = [&](auto Hc, const Raw &r) {
-        constexpr int H = decltype(Hc)::value;
-        // the 6-bit scales and mins (ggml get_scale_min_k4), four per dword
-        const uint32_t S0 = r.hdr[1], S1 = r.hdr[2], S2 = r.hdr[3];
-        const uint32_t scw = H == 0 ? (S0 & 0x3F3F3F3Fu) : ((S2 & 0x0F0F0F0Fu) | ((S0 >> 2) & 0x30303030u));
-        const int sh = 16 * (qp >> 2);
-        const half_t sc_lo = (half_t)(float)((scw >> sh) & 0xFFu);
-        const half_t sc_hi = (half_t)(float)((scw >> (sh + 8)) & 0xFFu);
-        const uint4_t wlo = qk_scaled8(r.q[0] & 0x0F0F0F0Fu, r.q[1] & 0x0F0F0F0Fu, sc_lo);
-        const uint4_t whi = qk_scaled8((r.q[0] >> 4) & 0x0F0F0F0Fu, (r.q[1] >> 4) & 0x0F0F0F0Fu, sc_hi);
-        half_t *dst = Ws + H * QK_WS + qrow * QK_WLD + 64 * (qp >> 2) + 8 * (qp & 3);
-        *(uint4_t *)dst = wlo, *(uint4_t *)(dst + 32) = whi;
-        if constexpr (H == 1) {
-            // the super-block's scalars travel with its second half; the eight threads of a row all store the
-            // same values (a branch for one of them would make the compiler wait for every load in flight)
-            const uint32_t mn03 = S1 & 0x3F3F3F3Fu;
-            const uint32_t mn47 = ((S2 >> 4) & 0x0F0F0F0Fu) | ((S1 >> 2) & 0x30303030u);
-            const half2_t dm = __builtin_bit_cast(half2_t, r.hdr[0]);
-            half2_t m0, m1, m2, m3;
-            qk_bytes_to_biased(mn03, m0, m1);
-            qk_bytes_to_biased(mn47, m2, m3);
-            const half2_t k = {(half_t)1024.0f, (half_t)1024.0f};
-            m0 -= k, m1 -= k, m2 -= k, m3 -= k;
-            Ds[qrow] = (float)dm[0], Dm[qrow] = (float)dm[1];
-            *(uint4_t *)(Mn + qrow * 8) = uint4_t{__builtin_bit_cast(uint32_t, m0), __builtin_bit_cast(uint32_t, m1),
-                                                  __builtin_bit_cast(uint32_t, m2), __builtin_bit_cast(uint32_t, m3)};
+    // ---- multiplying wavefront `wave`: weight rows i0 + 32 wave .. + 31.  Rows past the end repeat the last
+    // valid one.  Offsets are 32-bit from wave-uniform bases (the launcher checks the ranges).
+    struct Raw {
+        uint4_t hdr, qa, qb;
+    };
+    uint32_t woff[TA];
+#pragma unroll
+    for (int a = 0; a < TA; a++) woff[a] = (uint32_t)min(i0 + wave * 32 + 16 * a + fr, g.M - 1) * (uint32_t)g.nsb * 144u;
+    auto load_raw = [&](int64_t sb, Raw (&r)[TA]) {
+        const uint8_t *bsb = blocks + sb * 144; // wave-uniform
+#pragma unroll
+        for (int a = 0; a < TA; a++) {
+            r[a].hdr = *(const uint4_t *)(bsb + woff[a]);
+            r[a].qa = *(const uint4_t *)(bsb + (woff[a] + 16u + 32u * (uint32_t)fg));
+            r[a].qb = *(const uint4_t *)(bsb + (woff[a] + 32u + 32u * (uint32_t)fg));
         }
     };
-    // This wavefront's LDS stores of the tile about to be multiplied are done (its loads of raw blocks stay
-    // in flight: they are waited for where they are decoded); past the barrier the tile is whole, the
-    // loading wavefront having waited for its slots, and the stages of the tile before are free.
+    // what a thread keeps of a super-block's header: the scale pairs for its two sub-blocks as FMA operands,
+    // and for the min term (a super-block late) d, dmin and the two mins as f16 integers
+    struct Scl {
+        half2_t s_lo, n_lo, s_hi, n_hi;
+    };
+    struct Fin {
+        float d, dmin;
+        uint32_t mn;
+    };
+    const int sh = 16 * (fg & 1);
+    const uint32_t upper = (fg & 2) ? ~0u : 0u; // sub-blocks 4..7: the scales and mins split over two bytes
+    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    auto header = [&](const Raw &r, Scl &sc, Fin &f) {
+        // the 6-bit scales and mins (ggml get_scale_min_k4), four per dword; this thread's are 2 fg, 2 fg + 1
+        const uint32_t S0 = r.hdr[1], S1 = r.hdr[2], S2 = r.hdr[3];
+        const uint32_t sc47 = (S2 & 0x0F0F0F0Fu) | ((S0 >> 2) & 0x30303030u), mn47 = ((S2 >> 4) & 0x0F0F0F0Fu) | ((S1 >> 2) & 0x30303030u);
+        const uint32_t scw = (sc47 & upper) | (S0 & 0x3F3F3F3Fu & ~upper); // no branch: a divergent one makes the compiler wait for every load
+        const uint32_t mnw = (mn47 & upper) | (S1 & 0x3F3F3F3Fu & ~upper);
+        const half2_t s2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, scw >> sh, 0x04010400u)) - k1024;
+        const half2_t m2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, mnw >> sh, 0x04010400u)) - k1024;
+        const half_t lo = s2[0], hi = s2[1] * (half_t)0.0625f;
+        sc.s_lo = half2_t{lo, lo}, sc.s_hi = half2_t{hi, hi};
+        sc.n_lo = sc.s_lo * (half_t)-1024.0f, sc.n_hi = sc.s_hi * (half_t)-1024.0f;
+        const half2_t dm = __builtin_bit_cast(half2_t, r.hdr[0]);
+        f.d = (float)dm[0], f.dmin = (float)dm[1], f.mn = __builtin_bit_cast(uint32_t, m2);
+    };
+    // weight fragment of step T: 8 values sc * q of this thread's row
+    auto wfrag = [&](auto Tc, const Raw &r, const Scl &sc) {
+        constexpr int T = decltype(Tc)::value;
+        const uint4_t &q = (T & 2) ? r.qb : r.qa;
+        const uint32_t mask = T < 4 ? 0x0F0F0F0Fu : 0xF0F0F0F0u;
+        const uint32_t v0 = q[2 * (T & 1)] & mask, v1 = q[2 * (T & 1) + 1] & mask;
+        const half2_t s2 = T < 4 ? sc.s_lo : sc.s_hi, n2 = T < 4 ? sc.n_lo : sc.n_hi;
+        half2_t a = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v0, 0x04010400u));
+        half2_t bb = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v0, 0x04030402u));
+        half2_t c = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v1, 0x04010400u));
+        half2_t d = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v1, 0x04030402u));
+        a = __builtin_elementwise_fma(a, s2, n2), bb = __builtin_elementwise_fma(bb, s2, n2);
+        c = __builtin_elementwise_fma(c, s2, n2), d = __builtin_elementwise_fma(d, s2, n2);
+        return __builtin_bit_cast(half8_t, uint4_t{__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, bb),
+                                                   __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d)});
+    };
+    // This wavefront's LDS stores (its sums of x) are done; past the barrier the next activation tile is whole,
+    // the loading wavefront having waited for its slots, the stage of the tile before is free, and every
+    // wavefront's sums of the super-block before are visible.
     auto tile_ready = [&]() {
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
@@ -188,120 +200,164 @@ __global__ __launch_bounds__(QK_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
         asm volatile("" ::: "memory");
     };
 
-    float4_t acc[TA][TB], P[TA][TB];
-    float S[TB][8];
+    float4_t acc[TA][TB], P[2][TA][TB];
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int a = 0; a < TA; a++)
 #pragma unroll
-        for (int b = 0; b < TB; b++) acc[a][b] = zero, P[a][b] = zero;
-    const half8_t ones = {(half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1, (half_t)1};
+        for (int bq = 0; bq < TB; bq++) acc[a][bq] = zero, P[1][a][bq] = zero;
+    Fin fin[2][TA];
+#pragma unroll
+    for (int a = 0; a < TA; a++) fin[1][a] = Fin{0.f, 0.f, 0u};
+    // activation fragment bq of this wavefront is rows 16 ((bq + wave) % 4) .. + 15 of the tile, so that its
+    // fragment 0, the one it sums, is fragment `wave`
+    const uint32_t xlane = (uint32_t)(QR_ROWB * fr + 128 * fg);
+    uint2_t *sx_mine = Sx + (16 * wave + fr) * 4 + fg;
+    sx_mine[QR_BN * 4] = uint2_t{0u, 0u}; // parity 1 is read (against zero mins) under super-block 0
+    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
 
-    // MFMAs of the tile in stage H; `between` (the decoding of the next tile) is placed among them
-    auto compute = [&](auto Hc, int xst, auto &&between) {
-        constexpr int H = decltype(Hc)::value;
-        const half_t *wrow = Ws + H * QK_WS + (wi * 32 + fr) * QK_WLD + 8 * fg;
-        const half_t *xrow = Xs + xst * QK_XS + (wj * 32 + fr) * QK_KT;
-        auto sub_block = [&](int j) {
-            half8_t wf[TA], xf[TB];
+    // The min term of the super-block before (parity Q) and its fold into the accumulators.
+    auto read_sums = [&](int Q, uint2_t (&hl)[TB]) {
 #pragma unroll
-            for (int a = 0; a < TA; a++) wf[a] = __builtin_bit_cast(half8_t, *(const uint4_t *)(wrow + a * 16 * QK_WLD + 32 * j));
+        for (int bq = 0; bq < TB; bq++) hl[bq] = Sx[Q * QR_BN * 4 + (16 * ((bq + wave) & 3) + fr) * 4 + fg];
+    };
+    auto finish = [&](auto Qc, const uint2_t (&hl)[TB]) {
+        constexpr int Q = decltype(Qc)::value;
 #pragma unroll
-            for (int b = 0; b < TB; b++) xf[b] = __builtin_bit_cast(half8_t, *(const uint4_t *)(xrow + b * 16 * QK_KT + 8 * ((4 * j + fg) ^ fr)));
+        for (int bq = 0; bq < TB; bq++) {
+            const half8_t sf = __builtin_bit_cast(half8_t, uint4_t{hl[bq][0], hl[bq][1], 0u, 0u});
+#pragma unroll
+            for (int a = 0; a < TA; a++) {
+                const half8_t mf = __builtin_bit_cast(half8_t, uint4_t{fin[Q][a].mn, fin[Q][a].mn, 0u, 0u});
+                const float4_t T = __builtin_amdgcn_mfma_f32_16x16x32_f16(sf, mf, zero, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[a][bq][r] = fmaf(-fin[Q][a].dmin, T[r], fmaf(fin[Q][a].d, P[Q][a][bq][r], acc[a][bq][r]));
+            }
+        }
+    };
+
+    // One super-block of parity Pc: `cur` holds its raw blocks (loaded a super-block ago), `nxt` is the register
+    // set that the super-block before has left.
+    int xcur = 0;
+    auto step = [&](auto Pc, int64_t sb, const Raw (&cur)[TA], Raw (&nxt)[TA]) {
+        constexpr int PP = decltype(Pc)::value;
+        tile_ready();
+        load_raw(min(sb + 1, last), nxt);
+        uint2_t hl[TB];
+        read_sums(PP ^ 1, hl);
+        __builtin_amdgcn_sched_barrier(0); // the loads stay here, a super-block ahead of their decoding
+        Scl sc[TA];
+#pragma unroll
+        for (int a = 0; a < TA; a++) header(cur[a], sc[a], fin[PP][a]);
+        finish(std::integral_constant<int, PP ^ 1>{}, hl);
+        uint32_t xb[TB];
+#pragma unroll
+        for (int bq = 0; bq < TB; bq++) xb[bq] = xlane + (uint32_t)(xcur * QR_XSB + 16 * QR_ROWB * ((bq + wave) & 3));
+        float S0 = 0.f, S1 = 0.f;
+        auto xread = [&](int T, half8_t (&xf)[TB]) {
+#pragma unroll
+            for (int bq = 0; bq < TB; bq++) xf[bq] = __builtin_bit_cast(half8_t, *(const uint4_t *)(Xs + xb[bq] + 16 * T));
+        };
+        half8_t xf[2][TB];
+        xread(0, xf[0]);
+        // The order inside a super-block is the compiler's: pinning the fragment reads a step ahead of their MFMAs, or
+        // spreading them one per two MFMAs, measured the same or slower.
+        auto mfma_step = [&](auto Tc) {
+            constexpr int T = decltype(Tc)::value;
+            if constexpr (T < 7) xread(T + 1, xf[(T + 1) & 1]);
+            half8_t wf[TA];
+#pragma unroll
+            for (int a = 0; a < TA; a++) wf[a] = wfrag(Tc, cur[a], sc[a]);
 #pragma unroll
             for (int a = 0; a < TA; a++)
 #pragma unroll
-                for (int b = 0; b < TB; b++) // a super-block's first MFMA starts from zero: no clearing of P between super-blocks
-                    P[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[b], wf[a], (H == 0 && j == 0) ? zero : P[a][b], 0, 0, 0);
-            // sum of x over this sub-block for activation row lane % 16 (every register of the result holds it)
+                for (int bq = 0; bq < TB; bq++) // a super-block's first MFMA starts from zero: no clearing of P between super-blocks
+                    P[PP][a][bq] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[T & 1][bq], wf[a], T == 0 ? zero : P[PP][a][bq], 0, 0, 0);
+            const half8_t xs0 = xf[T & 1][0];
+            float &S = T < 4 ? S0 : S1;
 #pragma unroll
-            for (int b = 0; b < TB; b++) S[b][4 * H + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, xf[b], zero, 0, 0, 0)[0];
+            for (int c = 0; c < 4; c++) S = __builtin_amdgcn_fdot2(half2_t{xs0[2 * c], xs0[2 * c + 1]}, ones, S, false);
         };
-        sub_block(0);
-        sub_block(1);
-        between();
-        sub_block(2);
-        sub_block(3);
-        // three vector instructions of the decoding behind every MFMA of the second pair of sub-blocks
-#pragma unroll
-        for (int i = 0; i < 2 * (TA * TB + TB); i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-        }
+        mfma_step(std::integral_constant<int, 0>{});
+        mfma_step(std::integral_constant<int, 1>{});
+        mfma_step(std::integral_constant<int, 2>{});
+        mfma_step(std::integral_constant<int, 3>{});
+        mfma_step(std::integral_constant<int, 4>{});
+        mfma_step(std::integral_constant<int, 5>{});
+        mfma_step(std::integral_constant<int, 6>{});
+        mfma_step(std::integral_constant<int, 7>{});
+        // high part: the sum truncated to f16 (any f16 near it will do); low part: the exact remainder, rounded
+        const half2_t h = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(S0, S1));
+        const half2_t l = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(S0 - (float)h[0], S1 - (float)h[1]));
+        sx_mine[PP * QR_BN * 4] = uint2_t{__builtin_bit_cast(uint32_t, h), __builtin_bit_cast(uint32_t, l)};
+        xcur = xcur == QR_XST - 1 ? 0 : xcur + 1;
     };
 
-    // One tile: H = kt % 2 is its half of the super-block and its weight stage; `dec` holds the raw block of
-    // tile kt + 1 (loaded a step ago), `ld` is the register set that tile kt's raw block has left.
-    int xcur = 0;
-    auto step = [&](auto Hc, int64_t kt, const Raw &dec, Raw &ld) {
-        constexpr int H = decltype(Hc)::value;
-        tile_ready();
-        load_raw(min(kt + 2, last), ld); // past the end: the last tile again, decoded into a stage nobody reads
-        __builtin_amdgcn_sched_barrier(0); // the loads stay here, a tile and a half ahead of their decoding
-        compute(Hc, xcur, [&]() { decode_store(std::integral_constant<int, H ^ 1>{}, dec); });
-        xcur = xcur == QK_XST - 1 ? 0 : xcur + 1;
-    };
-    // The min term of a super-block whose two halves have been multiplied: K slots 0..7 (lane group 0) hold
-    // the eight sub-block sums, high parts then low parts in a second MFMA, against the eight integer mins;
-    // the mins of the other lane groups are zero, so whatever (finite) values their sum slots hold
-    // contributes nothing.
-    const uint32_t first_group = fg == 0 ? ~0u : 0u;
-    auto finish_super_block = [&]() {
-        half8_t mf[TA];
-        float d[TA], dmin[TA];
-#pragma unroll
-        for (int a = 0; a < TA; a++) {
-            const int row = wi * 32 + 16 * a + fr;
-            const uint4_t m = *(const uint4_t *)(Mn + row * 8);
-            mf[a] = __builtin_bit_cast(half8_t, uint4_t{m[0] & first_group, m[1] & first_group, m[2] & first_group, m[3] & first_group});
-            d[a] = Ds[row], dmin[a] = Dm[row];
-        }
-#pragma unroll
-        for (int b = 0; b < TB; b++) {
-            // high part: the sum truncated to f16 (any f16 near it will do); low part: the exact remainder, rounded
-            half8_t sh, sl;
-#pragma unroll
-            for (int j = 0; j < 8; j += 2) {
-                const half2_t h = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(S[b][j], S[b][j + 1]));
-                const half2_t l = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(S[b][j] - (float)h[0], S[b][j + 1] - (float)h[1]));
-                sh[j] = h[0], sh[j + 1] = h[1], sl[j] = l[0], sl[j + 1] = l[1];
-            }
-#pragma unroll
-            for (int a = 0; a < TA; a++) {
-                float4_t T = __builtin_amdgcn_mfma_f32_16x16x32_f16(sh, mf[a], zero, 0, 0, 0);
-                T = __builtin_amdgcn_mfma_f32_16x16x32_f16(sl, mf[a], T, 0, 0, 0);
-#pragma unroll
-                for (int r = 0; r < 4; r++) acc[a][b][r] = fmaf(-dmin[a], T[r], fmaf(d[a], P[a][b][r], acc[a][b][r]));
-            }
-        }
-    };
-
-    Raw r0, r1;
+    Raw r0[TA], r1[TA];
     load_raw(0, r0);
-    load_raw(1, r1);
-    decode_store(std::integral_constant<int, 0>{}, r0);
-    // a super-block per trip, one straight run of instructions (a branch inside it makes the compiler wait
+    // two super-blocks per trip, one straight run of instructions (a branch inside it makes the compiler wait
     // for every load in flight)
-    for (int64_t sb = 0; sb < g.nsb; sb++) {
-        step(std::integral_constant<int, 0>{}, 2 * sb, r1, r0);
-        step(std::integral_constant<int, 1>{}, 2 * sb + 1, r0, r1);
-        finish_super_block();
+    int64_t sb = 0;
+    for (; sb + 1 < g.nsb; sb += 2) {
+        step(std::integral_constant<int, 0>{}, sb, r0, r1);
+        step(std::integral_constant<int, 1>{}, sb + 1, r1, r0);
+    }
+    uint2_t hl[TB];
+    if (sb < g.nsb) {
+        step(std::integral_constant<int, 0>{}, sb, r0, r1);
+        tile_ready();
+        read_sums(0, hl);
+        finish(std::integral_constant<int, 0>{}, hl);
+    } else {
+        tile_ready();
+        read_sums(1, hl);
+        finish(std::integral_constant<int, 1>{}, hl);
     }
 
-    // acc[a][b][r]: weight row i0 + wi 32 + 16 a + fr, activation row j0 + wj 32 + 16 b + 4 fg + r
+    // acc[a][bq][r]: weight row i0 + 32 wave + 16 a + fr, activation row j0 + 16 ((bq + wave) % 4) + 4 fg + r
     half_t *out = g.out + s * g.o_bs;
+    if (vec_out) {
+        // Output contiguous along the weight rows: the tile goes through LDS (the activation stages are free: every
+        // wavefront's last fragment read and the last LDS-DMA lie before the barrier above) and leaves as 16-byte
+        // stores, 256 bytes per activation row.
+        constexpr int OLD = QR_BM + 8; // halfs per staged row: rows 272 bytes apart spread the lane groups over the banks
+        half_t *Os = (half_t *)smem;
+        rt_with_act(g.act, [&](auto has_act) {
+#pragma unroll
+            for (int a = 0; a < TA; a++) {
+                const int il = wave * 32 + 16 * a + fr;
+                const float bi = (g.has_bias && g.bias_on_rows) ? (float)g.bias[i0 + il] : 0.f;
+#pragma unroll
+                for (int bq = 0; bq < TB; bq++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int jl = 16 * ((bq + wave) & 3) + 4 * fg + r;
+                        float v = acc[a][bq][r] + bi;
+                        if (g.has_bias && !g.bias_on_rows) v += (float)g.bias[min(j0 + jl, g.N - 1)];
+                        Os[jl * OLD + il] = (half_t)rt_act_k<decltype(has_act)::value>(v);
+                    }
+            }
+        });
+        tile_ready();
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int row = (t >> 4) + 16 * k, c = t & 15;
+            if (j0 + row < g.N) *(uint4_t *)(out + (j0 + row) * g.o_js + i0 + 8 * c) = *(const uint4_t *)(Os + row * OLD + 8 * c);
+        }
+        return;
+    }
     rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
         for (int a = 0; a < TA; a++) {
-            const int64_t i = i0 + wi * 32 + 16 * a + fr;
+            const int64_t i = i0 + wave * 32 + 16 * a + fr;
             if (i >= g.M) continue;
 #pragma unroll
-            for (int b = 0; b < TB; b++)
+            for (int bq = 0; bq < TB; bq++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int64_t j = j0 + wj * 32 + 16 * b + 4 * fg + r;
+                    const int64_t j = j0 + 16 * ((bq + wave) & 3) + 4 * fg + r;
                     if (j >= g.N) continue;
-                    float v = acc[a][b][r];
+                    float v = acc[a][bq][r];
                     if (g.has_bias) v += (float)g.bias[g.bias_on_rows ? i : j];
                     v = rt_act_k<decltype(has_act)::value>(v);
                     out[i * g.o_is + j * g.o_js] = (half_t)v;
@@ -312,11 +368,10 @@ __global__ __launch_bounds__(QK_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
 
 RT_TUNABLE(g_gemm_q4k_disable, 0); // non-zero keeps Q4_K prefill on the generic kernel (for comparisons)
 
-// Q4_K weights (at least 64 rows) x K-contiguous f16 activations (more rows than one streaming launch
-// takes; up to 48 the dispatch tries a streaming launch per 16 first).  hipErrorNotSupported: another
-// kernel must take the problem.
+// Q4_K weights x K-contiguous f16 activations, more rows than one streaming launch takes.
+// hipErrorNotSupported: another kernel must take the problem.
 hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
-                           const DeviceInfo &) {
+                               const DeviceInfo &) {
     if (g_gemm_q4k_disable || p.a_dt != RT_Q4_K || p.act_dt != RT_F16) return hipErrorNotSupported;
     if (p.K % 256 != 0 || p.K < 256 || p.b_ks != 1 || p.M < 64 || p.N < 17 || p.stacks > 65535) return hipErrorNotSupported;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (p.b_js * 2) % 16 || (p.b_bs * 2) % 16) return hipErrorNotSupported;
@@ -324,16 +379,18 @@ hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const
     if (p.M * (p.K / 256) * 144 >= (int64_t(1) << 32) || p.N * p.b_js >= (int64_t(1) << 31)) return hipErrorNotSupported;
     GemmQ4kArgs g{};
     g.blocks = (const uint8_t *)A, g.X = (const half_t *)B, g.bias = (const half_t *)bias, g.out = (half_t *)out;
-    g.M = p.M, g.N = p.N, g.K = p.K, g.nsb = p.K / 256;
+    g.M = p.M, g.N = p.N, g.nsb = p.K / 256;
     g.a_stack = p.a_stack, g.b_stack = p.b_stack;
     g.b_bs = p.b_bs, g.b_js = p.b_js;
     g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
-    const int64_t tiles_i = (p.M + QK_BM - 1) / QK_BM, tiles_j = (p.N + QK_BN - 1) / QK_BN;
+    const int64_t tiles_i = (p.M + QR_BM - 1) / QR_BM, tiles_j = (p.N + QR_BN - 1) / QR_BN;
     if (tiles_i * tiles_j > 0x7fffffff) return hipErrorNotSupported;
     g.tiles_j = (int)tiles_j;
+    g.remap = (tiles_i * tiles_j) % 8 == 0;
+    g.vec_out = p.o_is == 1 && p.o_js % 8 == 0 && p.o_bs % 8 == 0 && ((uintptr_t)out & 15u) == 0;
     if (const hipError_t e = ensure_lds_limit<&gemm_q4k_kernel>(); e != hipSuccess) return e;
-    hipLaunchKernelGGL(gemm_q4k_kernel, dim3((unsigned)(tiles_i * tiles_j), (unsigned)p.stacks), dim3(QK_THREADS), QK_LDS, stream, g);
+    hipLaunchKernelGGL(gemm_q4k_kernel, dim3((unsigned)(tiles_i * tiles_j), (unsigned)p.stacks), dim3(QR_THREADS), QR_LDS, stream, g);
     return hipGetLastError();
 }
 
