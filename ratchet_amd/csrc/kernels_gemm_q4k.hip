@@ -57,18 +57,21 @@ struct GemmQ4kArgs {
     int has_bias, bias_on_rows, act;
 };
 
-constexpr int QR_BM = 128, QR_BN = 64; // weight rows x activation rows per workgroup
+constexpr int QR_BN = 64; // activation rows per workgroup; weight rows: 16 per MFMA tile x TA tiles x MW multiplying wavefronts
 // An activation stage holds one super-block of K for 64 rows: 32 K-vectors of 16 bytes per row and one of padding,
 // so that the 16 rows of a fragment read start 4 banks apart and a read address is base + 16 * step.
 constexpr int QR_ROWB = 33 * 16;       // bytes per staged row
 constexpr int QR_XSB = QR_BN * QR_ROWB; // bytes per stage = 33 LDS-DMA instructions of 1 KB
 constexpr int QR_XST = 3;              // activation stages: a tile's slots are in flight for two super-blocks
 constexpr int QR_LW = 4;               // wavefronts that only issue the LDS-DMA, one per SIMD
-constexpr int QR_THREADS = 256 + 64 * QR_LW;
 constexpr size_t QR_LDS = (size_t)QR_XST * QR_XSB + 2 * QR_BN * 4 * 8;
 
-__global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
-    constexpr int TA = 2, TB = 4; // MFMA tiles per wavefront: weight rows (second operand), activation rows (first)
+// TA: MFMA tiles of weight rows per wavefront; MW: multiplying wavefronts (4: each sums the activation fragment of its number)
+template <int TA, int MW>
+__global__ __launch_bounds__(64 * (MW + QR_LW)) void gemm_q4k_kernel(GemmQ4kArgs g) {
+    constexpr int TB = 4;             // MFMA tiles per wavefront: TA of weight rows (second operand), TB of activation rows (first)
+    constexpr int BM = 16 * TA * MW;  // weight rows per workgroup
+    static_assert(MW == 4, "wavefront w sums the x of activation fragment w: four fragments, four wavefronts");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t *Xs = smem;                             // [QR_XST][64 rows][33 slots of 16 bytes]: K-vector v of row r in slot v
     uint2_t *Sx = (uint2_t *)(Xs + QR_XST * QR_XSB); // [2][64][4]: sums of x of super-block parity p, row, lane group: (high pair, low pair)
@@ -82,18 +85,18 @@ __global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
     uint32_t b = blockIdx.x;
     if (g.remap) b = (b & 7) * (gridDim.x >> 3) + (b >> 3);
     const uint32_t ti = b / (uint32_t)g.tiles_j, tj = b - ti * (uint32_t)g.tiles_j;
-    const int64_t i0 = (int64_t)ti * QR_BM, j0 = (int64_t)tj * QR_BN;
+    const int64_t i0 = (int64_t)ti * BM, j0 = (int64_t)tj * QR_BN;
     const uint8_t *blocks = g.blocks + (g.a_stack == 1 ? 0 : s) * g.M * g.nsb * 144;
     const half_t *X = g.X + (g.b_stack == 1 ? 0 : s) * g.b_bs;
     const int64_t last = g.nsb - 1;
-    const bool vec_out = g.vec_out && i0 + QR_BM <= g.M; // a whole tile of weight rows, stored 16 bytes at a time
+    const bool vec_out = g.vec_out && i0 + BM <= g.M; // a whole tile of weight rows, stored 16 bytes at a time
 
-    if (wave >= 4) {
+    if (wave >= MW) {
         // ---- loading wavefront lw: LDS-DMA instruction i of a stage (i = lw, lw + 4, ...; 33 in all) fills the 1 KB
         // run of slots 64 i .. + 63; slot p is K-vector p % 33 of row p / 33 (the 33rd is padding and repeats the 32nd).
         // Each of the four issues nine: the ninth of wavefronts 1..3 repeats instruction 32.
         constexpr int NI = 9;
-        const int lw = wave - 4;
+        const int lw = wave - MW;
         uint32_t xsrc[NI];
 #pragma unroll
         for (int n = 0; n < NI; n++) {
@@ -138,7 +141,7 @@ __global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
     };
     uint32_t woff[TA];
 #pragma unroll
-    for (int a = 0; a < TA; a++) woff[a] = (uint32_t)min(i0 + wave * 32 + 16 * a + fr, g.M - 1) * (uint32_t)g.nsb * 144u;
+    for (int a = 0; a < TA; a++) woff[a] = (uint32_t)min(i0 + wave * (16 * TA) + 16 * a + fr, g.M - 1) * (uint32_t)g.nsb * 144u;
     auto load_raw = [&](int64_t sb, Raw (&r)[TA]) {
         const uint8_t *bsb = blocks + sb * 144; // wave-uniform
 #pragma unroll
@@ -320,12 +323,12 @@ __global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
         // Output contiguous along the weight rows: the tile goes through LDS (the activation stages are free: every
         // wavefront's last fragment read and the last LDS-DMA lie before the barrier above) and leaves as 16-byte
         // stores, 256 bytes per activation row.
-        constexpr int OLD = QR_BM + 8; // halfs per staged row: rows 272 bytes apart spread the lane groups over the banks
+        constexpr int OLD = BM + 8; // halfs per staged row: rows 272 bytes apart spread the lane groups over the banks
         half_t *Os = (half_t *)smem;
         rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
             for (int a = 0; a < TA; a++) {
-                const int il = wave * 32 + 16 * a + fr;
+                const int il = wave * (16 * TA) + 16 * a + fr;
                 const float bi = (g.has_bias && g.bias_on_rows) ? (float)g.bias[i0 + il] : 0.f;
 #pragma unroll
                 for (int bq = 0; bq < TB; bq++)
@@ -340,8 +343,9 @@ __global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
         });
         tile_ready();
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int row = (t >> 4) + 16 * k, c = t & 15;
+        for (int k = 0; k < 2 * TA; k++) {
+            constexpr int CPR = BM / 8; // 16-byte pieces per row
+            const int idx = t + 64 * MW * k, row = idx / CPR, c = idx % CPR;
             if (j0 + row < g.N) *(uint4_t *)(out + (j0 + row) * g.o_js + i0 + 8 * c) = *(const uint4_t *)(Os + row * OLD + 8 * c);
         }
         return;
@@ -349,7 +353,7 @@ __global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
     rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
         for (int a = 0; a < TA; a++) {
-            const int64_t i = i0 + wave * 32 + 16 * a + fr;
+            const int64_t i = i0 + wave * (16 * TA) + 16 * a + fr;
             if (i >= g.M) continue;
 #pragma unroll
             for (int bq = 0; bq < TB; bq++)
@@ -366,12 +370,13 @@ __global__ __launch_bounds__(QR_THREADS) void gemm_q4k_kernel(GemmQ4kArgs g) {
     });
 }
 
+RT_TUNABLE(g_gemm_q4k_cfg, 0); // 14 / 24: always one / two weight tiles per wavefront (for comparisons)
 RT_TUNABLE(g_gemm_q4k_disable, 0); // non-zero keeps Q4_K prefill on the generic kernel (for comparisons)
 
 // Q4_K weights x K-contiguous f16 activations, more rows than one streaming launch takes.
 // hipErrorNotSupported: another kernel must take the problem.
 hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
-                               const DeviceInfo &) {
+                           const DeviceInfo &dev) {
     if (g_gemm_q4k_disable || p.a_dt != RT_Q4_K || p.act_dt != RT_F16) return hipErrorNotSupported;
     if (p.K % 256 != 0 || p.K < 256 || p.b_ks != 1 || p.M < 64 || p.N < 17 || p.stacks > 65535) return hipErrorNotSupported;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (p.b_js * 2) % 16 || (p.b_bs * 2) % 16) return hipErrorNotSupported;
@@ -384,14 +389,24 @@ hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const
     g.b_bs = p.b_bs, g.b_js = p.b_js;
     g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
-    const int64_t tiles_i = (p.M + QR_BM - 1) / QR_BM, tiles_j = (p.N + QR_BN - 1) / QR_BN;
-    if (tiles_i * tiles_j > 0x7fffffff) return hipErrorNotSupported;
+    const int64_t tiles_j = (p.N + QR_BN - 1) / QR_BN;
     g.tiles_j = (int)tiles_j;
-    g.remap = (tiles_i * tiles_j) % 8 == 0;
     g.vec_out = p.o_is == 1 && p.o_js % 8 == 0 && p.o_bs % 8 == 0 && ((uintptr_t)out & 15u) == 0;
-    if (const hipError_t e = ensure_lds_limit<&gemm_q4k_kernel>(); e != hipSuccess) return e;
-    hipLaunchKernelGGL(gemm_q4k_kernel, dim3((unsigned)(tiles_i * tiles_j), (unsigned)p.stacks), dim3(QR_THREADS), QR_LDS, stream, g);
-    return hipGetLastError();
+    auto go = [&](auto kernel, int bm, int threads) -> hipError_t {
+        const int64_t tiles_i = (p.M + bm - 1) / bm;
+        if (tiles_i * tiles_j > 0x7fffffff) return hipErrorNotSupported;
+        g.remap = (tiles_i * tiles_j) % 8 == 0;
+        if (const hipError_t e = ensure_lds_limit<decltype(kernel)::value>(); e != hipSuccess) return e;
+        hipLaunchKernelGGL(decltype(kernel)::value, dim3((unsigned)(tiles_i * tiles_j), (unsigned)p.stacks), dim3(threads), QR_LDS, stream, g);
+        return hipGetLastError();
+    };
+    // Four multiplying wavefronts of 32 weight rows x 64 activation rows each; when the grid of 16-row wavefronts
+    // (64 weight rows per workgroup) still fits the compute units in one round, those: half the work per wavefront
+    // (8192 x 3072 at 64 / 128 rows: 15.7 / 16.8 us against 22.6 / 23.6; 3072 x 8192 at 256 rows: 35 against 52 us).
+    const int64_t wgs_small = ((p.M + 63) / 64) * tiles_j;
+    const bool small = g_gemm_q4k_cfg == 14 || (g_gemm_q4k_cfg == 0 && wgs_small <= dev.num_cus);
+    if (small) return go(std::integral_constant<void (*)(GemmQ4kArgs), &gemm_q4k_kernel<1, 4>>{}, 64, 512);
+    return go(std::integral_constant<void (*)(GemmQ4kArgs), &gemm_q4k_kernel<2, 4>>{}, 128, 512);
 }
 
 } // namespace rt

@@ -285,13 +285,13 @@ RT_TUNABLE(g_gemv_disable_mfma, 0);
 // launch streams the weights again (after the first mostly from the Infinity Cache), which still beats
 // the tiled kernels while the MFMA work is small: measured at 10240 x 2560 Q8_0H, 17 / 32 / 48 / 64
 // vectors take 17 / 21 / 31 / 42 us against 34 / 35 / 35 / 51 us tiled, and at 8192 x 3072 Q4_K
-// 17 / 32 / 48 vectors take 14 / 18 / 27 us against 30 us tiled at any of them (56 vectors: 32 us,
-// and the tiled kernel takes over from 49).
+// 17 / 32 / 48 vectors take 12 / 14 / 21 us against 15 us tiled at any count up to 64: the tiled
+// kernel takes over from 33.
 hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                hipStream_t stream, const DeviceInfo &dev) {
     const bool q8 = p.a_dt == RT_Q8_0H, q4 = p.a_dt == RT_Q4_K;
     if ((!q8 && !q4) || p.act_dt != RT_F16 || g_gemv_disable_mfma) return hipErrorNotSupported;
-    if (p.N <= 16 || p.N > (q8 ? 64 : 48)) return hipErrorNotSupported;
+    if (p.N <= 16 || p.N > (q8 ? 64 : 32)) return hipErrorNotSupported;
     for (int64_t j0 = 0; j0 < p.N; j0 += 16) {
         Problem c = p;
         c.N = p.N - j0 < 16 ? p.N - j0 : 16;

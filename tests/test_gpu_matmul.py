@@ -796,14 +796,17 @@ def test_f32_contiguous_operands(device, oracle):
 
 
 # ---------------------------------------------------------------------------
-# Q4_K weights against 49 or more activation rows: the tiled kernel over half super-blocks
+# Q4_K weights against 33 or more activation rows: the tiled kernel that decodes the weights in registers
 # ---------------------------------------------------------------------------
 def test_q4k_prefill_tiles(device, oracle):
-    """Tile edges in both dimensions (64 weight rows x 128 activation rows per workgroup), one super-block
-    of K to many, per-stack activations against one weight, both bias axes, both output orientations."""
+    """Tile edges in both dimensions (64 or 128 weight rows x 64 activation rows per workgroup: the last two
+    shapes have more than 256 workgroups of 64 weight rows and take the 128-row form), one super-block of K to
+    many, per-stack activations against one weight, both bias axes, both output orientations (contiguous along
+    the weight rows: 16-byte stores through LDS, whole tiles only; the other: scalar stores)."""
     #        S  N(weight rows) M(activation rows) K
     shapes = [(1, 64, 64, 256), (1, 65, 129, 512), (1, 200, 100, 1024), (2, 130, 257, 768), (1, 1000, 70, 256),
-              (3, 96, 64, 2048), (1, 64, 700, 512), (1, 128, 49, 512), (2, 70, 63, 256), (1, 64, 96, 1280)]
+              (3, 96, 64, 2048), (1, 64, 700, 512), (1, 128, 49, 512), (2, 70, 63, 256), (1, 64, 96, 1280),
+              (1, 136, 33, 512), (1, 2100, 520, 512), (2, 2056, 530, 256)]
     for i, (S, N, M, K) in enumerate(shapes):
         rng = np.random.default_rng(1200 + i)
         blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
@@ -842,6 +845,17 @@ def test_q4k_prefill_one_hot_is_the_dequantized_weight(device, oracle):
     want = dq[:, cols].T.astype(np.float16)
     bad = np.argwhere(got[0].view(np.uint16) != want.view(np.uint16))
     assert bad.size == 0, (len(bad), bad[:8].tolist())
+    # the same through the form with 128 weight rows per workgroup (more than 256 workgroups of 64 rows)
+    N, K, M = 4200, 512, 300
+    blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    dq = oracle.q4k_dequantize(blocks).reshape(N, K)
+    cols = np.concatenate([np.arange(0, K, 19), rng.integers(0, K, size=M)])[:M]
+    x = np.zeros((1, M, K), dtype=np.float16)
+    x[0, np.arange(M), cols] = 1
+    got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (N, K)), Tensor.from_data(x), None, False, True, True)
+    want = dq[:, cols].T.astype(np.float16)
+    bad = np.argwhere(got[0].view(np.uint16) != want.view(np.uint16))
+    assert bad.size == 0, (len(bad), bad[:8].tolist())
 
 
 @pytest.mark.parametrize("M", [1, 16, 64, 256], ids=["streaming-1", "streaming-16", "tiled-64", "tiled-256"])
@@ -870,12 +884,12 @@ def test_q4k_known_answer_block_through_every_kernel(device, oracle, q4k_kat, M)
 
 
 # ---------------------------------------------------------------------------
-# 17..64 (Q8_0H) and 17..48 (Q4_K) activation vectors: one streaming launch per 16 of them
+# 17..64 (Q8_0H) and 17..32 (Q4_K) activation vectors: one streaming launch per 16 of them
 # ---------------------------------------------------------------------------
 def test_quantized_weights_a_few_more_vectors_than_one_streaming_launch(device, oracle):
     rng = np.random.default_rng(1100)
     cases = [("q8", 1, 512, 2560, m) for m in (17, 32, 48, 64)] + [("q8", 2, 96, 512, 33)] + \
-            [("q4k", 1, 256, 3072, m) for m in (17, 40, 48)] + [("q4k", 2, 64, 1024, 31)]
+            [("q4k", 1, 256, 3072, m) for m in (17, 32, 40, 48)] + [("q4k", 2, 64, 1024, 31)]
     for kind, S, N, K, M in cases:
         w = (rng.standard_normal((S, N, K)) * 0.05).astype(np.float32)
         if kind == "q8":
