@@ -491,13 +491,15 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
 #pragma unroll
     for (int i = 0; i < TM + TN; i++) read_one(0, 0, f0, i);
     int cur = 0, nxt = 1;
-    static_assert(TM * TN / 2 >= TM + TN, "not enough MFMAs to spread the reads over");
+    // a fragment read behind every second MFMA, or behind every one where the tile has too few of them
+    constexpr int RS = TM * TN / 2 >= TM + TN ? 2 : 1;
+    static_assert(TM * TN / RS >= TM + TN, "not enough MFMAs to spread the reads over");
     for (int64_t kt = 0; kt < nk; kt++) {
 #pragma unroll
         for (int m = 0; m < TM * TN; m++) {
             acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f0.fb[m % TN], f0.fa[m / TN], acc[m / TN][m % TN], 0, 0, 0);
-            if (m % 2 == 1) {
-                if (m / 2 < TM + TN) read_one(cur, 1, f1, m / 2);
+            if (m % RS == RS - 1) {
+                if (m / RS < TM + TN) read_one(cur, 1, f1, m / RS);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -505,8 +507,8 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
 #pragma unroll
         for (int m = 0; m < TM * TN; m++) {
             acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f1.fb[m % TN], f1.fa[m / TN], acc[m / TN][m % TN], 0, 0, 0);
-            if (m % 2 == 1) {
-                if (m / 2 < TM + TN) read_one(nxt, 0, f0, m / 2);
+            if (m % RS == RS - 1) {
+                if (m / RS < TM + TN) read_one(nxt, 0, f0, m / RS);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -913,6 +915,7 @@ static hipError_t launch_nt_dl(const GemmNtArgs &g, int64_t stacks, hipStream_t 
 // (3 or 4, 0 = 3) of the direct-to-LDS kernel (for comparisons).
 RT_TUNABLE(g_gemm_nt_no_direct, 0);
 RT_TUNABLE(g_gemm_nt_stages, 0);
+RT_TUNABLE(g_gemm_nt_narrow, 0); // 1: never the 64- and 96-row tiles for few activation rows (for comparisons)
 RT_TUNABLE(g_gemm_nt_shortk_parts, 0); // workgroups per strip of the short-K kernel (0 = automatic)
 
 template <int BM, int BN, bool Q8, bool KFULL>
@@ -963,7 +966,7 @@ static bool nt_orient(Problem &p) {
 uint64_t gemm_nt_workspace_bytes(const Problem &p0, const DeviceInfo &dev) {
     Problem p = p0;
     nt_orient(p);
-    if (p.a_ks != 1 || p.b_ks != 1 || p.M < 160 || p.N < 64) return 0;
+    if (p.a_ks != 1 || p.b_ks != 1 || p.M < 160 || p.N < 8) return 0;
     const int ks = gemm_nt_ksplit(p, dev);
     return ks > 1 ? (uint64_t)p.stacks * ks * p.M * p.N * sizeof(float) : 0;
 }
@@ -982,8 +985,9 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
     const bool q8 = p.a_dt == RT_Q8_0H;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (p.b_js * 2) % 16 || (p.b_bs * 2) % 16) return hipErrorNotSupported;
     if (q8 ? (p.K % 32 != 0) : ((p.a_rs * 2) % 16 != 0 || (p.a_bs * 2) % 16 != 0)) return hipErrorNotSupported;
-    // small problems do not fill the large tile; the 128 x 128 kernel handles them
-    if (p.M < 160 || p.N < 64) return hipErrorNotSupported;
+    // small problems do not fill the tiles; the generic kernel handles them (at 10240 x 2560 f16 weights it takes
+    // 19.7 us for 8 activation rows and 33 us for 16..48, the 64-row tiles here 17.4 us for any count up to 64)
+    if (p.M < 160 || p.N < 8) return hipErrorNotSupported;
 
     GemmNtArgs g{};
     g.A = A, g.B = (const half_t *)B, g.bias = (const half_t *)bias, g.out = (half_t *)out;
@@ -1025,6 +1029,12 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
     const int64_t ti = (p.M + BM - 1) / BM, tj = (p.N + BN - 1) / BN;
     if (ti * tj > 0x7fffffff) return hipErrorNotSupported;
     g.tiles_i = (int)ti, g.tiles_j = (int)tj;
+    // few activation rows: 160-row tiles leave most compute units idle and a workgroup takes as long for one
+    // column of tiles as for four; 64-row tiles, while all of them still run at once, put 2.5 times the workgroups to work
+    // (10240 x 2560 f16 weights: 65..128 rows 24.6-25.4 -> 17.2-18.1 us); 96-row tiles where those no longer fit.
+    const int64_t ti64 = (p.M + 63) / 64, ti96 = (p.M + 95) / 96;
+    const bool few = g_gemm_nt_narrow != 1 && ti * tj * p.stacks * 2 <= dev.num_cus;
+    const int bm = few && ti64 * tj * p.stacks <= dev.num_cus ? 64 : few && ti96 * tj * p.stacks <= dev.num_cus ? 96 : BM;
     const bool dl_f16 = !q8 && kfull && !g_gemm_nt_no_direct;
     const bool dl_q8 = q8 && p.K % 256 == 0 && !g_gemm_nt_no_direct && ((uintptr_t)g.scales & 15u) == 0 && (p.a_bs % 512) == 0;
     if (dl_f16 || dl_q8) {
@@ -1032,6 +1042,11 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
         if (ks > 1 && p.workspace && !((uintptr_t)p.workspace & 15u) &&
             p.workspace_bytes >= (uint64_t)p.stacks * ks * p.M * p.N * sizeof(float))
             g.ksplit = ks, g.k_len = p.K / ks, g.partial = (float *)p.workspace;
+    }
+    if ((dl_f16 || dl_q8) && bm != BM && g.ksplit == 1) {
+        g.tiles_i = (int)(bm == 64 ? ti64 : ti96);
+        if (dl_f16) return bm == 64 ? launch_nt_dl<64, BN, 3, 2>(g, p.stacks, stream) : launch_nt_dl<96, BN, 3, 2>(g, p.stacks, stream);
+        return bm == 64 ? launch_nt_q8w<64, BN, 4>(g, p.stacks, stream) : launch_nt_q8w<96, BN, 4>(g, p.stacks, stream);
     }
     if (dl_f16) {
         // two loading wavefronts: one and four measured the same within run-to-run spread

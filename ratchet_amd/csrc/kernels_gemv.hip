@@ -283,15 +283,14 @@ RT_TUNABLE(g_gemv_disable_mfma, 0);
 // such requirement.
 // A few more activation vectors than one streaming launch takes: one launch per 16 of them.  Each
 // launch streams the weights again (after the first mostly from the Infinity Cache), which still beats
-// the tiled kernels while the MFMA work is small: measured at 10240 x 2560 Q8_0H, 17 / 32 / 48 / 64
-// vectors take 17 / 21 / 31 / 42 us against 34 / 35 / 35 / 51 us tiled, and at 8192 x 3072 Q4_K
-// 17 / 32 / 48 vectors take 12 / 14 / 21 us against 15 us tiled at any count up to 64: the tiled
-// kernel takes over from 33.
+// the tiled kernels while the MFMA work is small: measured at 10240 x 2560 Q8_0H, 17 / 32 vectors take
+// 18 / 20 us (48 / 64: 29 / 38) against 21 us tiled at any count up to 64, and at 8192 x 3072 Q4_K
+// 17 / 32 vectors take 12 / 14 us (48: 21) against 15 us tiled: the tiled kernels take over from 33.
 hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                hipStream_t stream, const DeviceInfo &dev) {
     const bool q8 = p.a_dt == RT_Q8_0H, q4 = p.a_dt == RT_Q4_K;
     if ((!q8 && !q4) || p.act_dt != RT_F16 || g_gemv_disable_mfma) return hipErrorNotSupported;
-    if (p.N <= 16 || p.N > (q8 ? 64 : 32)) return hipErrorNotSupported;
+    if (p.N <= 16 || p.N > 32) return hipErrorNotSupported;
     for (int64_t j0 = 0; j0 < p.N; j0 += 16) {
         Problem c = p;
         c.N = p.N - j0 < 16 ? p.N - j0 : 16;

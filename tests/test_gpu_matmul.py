@@ -609,6 +609,21 @@ def test_f16_nt_gemm_edges(device, oracle, trans_out):
         check(oracle, got, want, DType.F16, (S, M, N, K, trans_out))
 
 
+def test_f16_weights_few_activation_rows(device, oracle):
+    """8..63 activation rows against f16 weights of 160 rows or more: the tiled kernel's 64-row tiles with a
+    mostly empty column of activation rows (fewer than 8 rows stay on the generic kernel)."""
+    for i, (M, N, K) in enumerate([(512, 8, 320), (700, 9, 128), (1000, 33, 512), (161, 63, 64), (2560, 17, 2560)]):
+        rng = np.random.default_rng(660 + i)
+        w = (rng.standard_normal((M, K)) * 0.05).astype(np.float16)
+        x = rng.standard_normal((1, N, K)).astype(np.float16)
+        for to in (True, False):
+            bias = rng.standard_normal(M if to else N).astype(np.float16) if (i + to) % 2 == 0 else None
+            got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x),
+                             None if bias is None else Tensor.from_data(bias), False, True, to)
+            want = oracle.matmul_ref(w, oracle.F16, w.shape, x, oracle.F16, x.shape, bias, False, True, to)
+            check(oracle, got, want, DType.F16, (M, N, K, to))
+
+
 def test_f16_nt_gemm_stack_broadcast(device, oracle):
     rng = np.random.default_rng(650)
     a = rng.standard_normal((1, 200, 128)).astype(np.float16)      # one weight, four activation stacks
@@ -641,7 +656,7 @@ def test_q8_tiled_one_hot_is_bit_exact_dequant(device, oracle):
     """The tiled Q8_0H kernels (K % 256 == 0 and not) with one-hot activations: each output is one
     dequantized weight, which must match the oracle's dequantizer bit for bit, -128 included."""
     rng = np.random.default_rng(720)
-    for N, K, M in [(320, 256, 64), (200, 512, 100), (170, 96, 70)]:
+    for N, K, M in [(320, 256, 64), (200, 512, 100), (170, 96, 70), (2100, 256, 1300), (9000, 256, 200)]:  # the last two: 160- and 96-row tiles
         buf = q8_weight(oracle, rng, N, K, DType.Q8_0H)
         buf[: N * K][3::89] = 0x80
         dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
@@ -884,7 +899,7 @@ def test_q4k_known_answer_block_through_every_kernel(device, oracle, q4k_kat, M)
 
 
 # ---------------------------------------------------------------------------
-# 17..64 (Q8_0H) and 17..32 (Q4_K) activation vectors: one streaming launch per 16 of them
+# 17..32 activation vectors against Q8_0H or Q4_K weights: one streaming launch per 16 of them (33..64: the tiled kernels)
 # ---------------------------------------------------------------------------
 def test_quantized_weights_a_few_more_vectors_than_one_streaming_launch(device, oracle):
     rng = np.random.default_rng(1100)
@@ -906,13 +921,16 @@ def test_quantized_weights_a_few_more_vectors_than_one_streaming_launch(device, 
             check(oracle, got, want, DType.F16, (kind, S, N, K, M, to))
 
 
-@pytest.mark.parametrize("rows_w,rows_x", [(1280, 768), (1280, 1408), (2560, 640)], ids=["8x6", "8x11", "16x5"])
+@pytest.mark.parametrize("rows_w,rows_x", [(1280, 768), (1280, 1408), (2560, 640), (2100, 1300), (9000, 200), (4100, 100)],
+                         ids=["8x6", "8x11", "16x5", "160-row-tiles-14x11-edges", "96-row-tiles", "64-row-tiles-edges"])
 @pytest.mark.parametrize("quant", [False, True], ids=["f16", "q8_0h"])
 def test_large_tile_panel_order(device, oracle, rows_w, rows_x, quant):
     """Large-tile NT GEMMs with whole weight row blocks per XCD and more than four activation column blocks walk
     their tiles in panels of four column blocks (a narrower last panel included): every output tile must be
-    written exactly once.  The output of each 160 x 128 tile depends on its position (distinct rows of both
-    operands), so a tile computed twice or never shows against the oracle."""
+    written exactly once.  The output of each tile depends on its position (distinct rows of both
+    operands), so a tile computed twice or never shows against the oracle.  A grid of 160-row tiles that would
+    leave half the compute units idle is cut into 64-row tiles, or 96-row ones where those no longer run all at
+    once: the ids name the form a shape takes on 256 compute units (the first three: 64-row tiles)."""
     rng = np.random.default_rng(rows_w + rows_x)
     K = 256
     w = (rng.standard_normal((rows_w, K)) * 0.05).astype(np.float32)
