@@ -93,7 +93,8 @@ class Runner:
         (ms_per_step, mode); `stats`, a dict, also receives the fastest and slowest region and the count.
         The launches are captured into one HIP graph of whole rotations of the weight copies (20 launches
         or more) when capture works, so the host's launch rate does not bound a ~6 us kernel; a region is
-        steps // 20 replays plus the remaining launches one by one.  Otherwise all are issued one by one."""
+        steps // 20 replays plus the remaining launches one by one, behind one untimed replay that keeps the
+        device busy while the host enqueues the region.  Otherwise all are issued one by one."""
         torch = self.torch
         for i in range(warmup):
             launch_step(i % n_variants)
@@ -116,6 +117,11 @@ class Runner:
         for _ in range(self.REGIONS):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
+            if graph is not None:
+                # one untimed replay ahead of the first event: the device is still busy with it while the host
+                # enqueues the event and the timed replays, so a short region (the driver's --steps 20 is a single
+                # replay) holds its `steps` launches back to back like a long one, not the host's enqueue latency too
+                graph.replay()
             e0.record()
             if graph is not None:
                 full, rest = divmod(steps, per_graph)
