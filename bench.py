@@ -628,6 +628,43 @@ def read_calibration(r: Runner, O, steps, warmup):
     return {"read_calibration": rows, "weight_copies_rotated": copies, "steps": steps, "regions": Runner.REGIONS}
 
 
+def issue_calibration(r: Runner):
+    """Context for the tiled kernels that decode or fold in their multiplying wavefronts: what MFMAs, packed vector
+    instructions and LDS fragment reads cost a wavefront alone and mixed.  One wavefront per SIMD on every compute
+    unit runs 4000 trips of (8 MFMAs, 8 x NV packed FMAs, ND fragment reads); ns per trip from HIP events around
+    one launch, median of 5.  The probe is in ratchet_amd/libratchet_probes.so (csrc/bench_probes.hip)."""
+    torch = r.torch
+    P = ctypes.CDLL(os.path.join(ROOT, "ratchet_amd", "libratchet_probes.so"))
+    vp = ctypes.c_void_p
+    P.probe_issue_mix.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+    src = torch.zeros(8192, dtype=torch.uint8, device="cuda:0")
+    dst = torch.zeros(256 * 1024, dtype=torch.uint8, device="cuda:0")
+    iters, rows = 4000, []
+    mixes = [("8 MFMAs", 0, 8, 0), ("24 packed FMAs", 3, 0, 0), ("8 MFMAs + 8 packed FMAs", 1, 8, 0),
+             ("8 MFMAs + 16 packed FMAs", 2, 8, 0), ("8 MFMAs + 24 packed FMAs", 3, 8, 0),
+             ("8 MFMAs + 32 packed FMAs", 4, 8, 0), ("8 MFMAs + 48 packed FMAs", 6, 8, 0),
+             ("8 MFMAs + 4 fragment reads", 0, 8, 4), ("24 packed FMAs + 4 fragment reads", 3, 0, 4),
+             ("8 MFMAs + 24 packed FMAs + 2 fragment reads", 3, 8, 2), ("8 MFMAs + 24 packed FMAs + 4 fragment reads", 3, 8, 4)]
+    for name, nv, nm, nd in mixes:
+        def launch():
+            rc = P.probe_issue_mix(nv, nm, nd, iters, vp(src.data_ptr()), vp(dst.data_ptr()), vp(torch.cuda.current_stream().cuda_stream))
+            if rc != 0:
+                raise RuntimeError(f"probe launch failed: hipError {rc}")
+        launch()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            launch()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e6 / iters)
+        ts.sort()
+        rows.append({"trip": name, "ns_per_trip": round(ts[2], 1)})
+    return {"issue_calibration": rows, "trips": iters, "wavefronts_per_simd": 1}
+
+
 def cpu_baseline(O, wbuf, x, bias, budget_s=1.5):
     """The oracle's reference path on the host cores, same inputs: median of >= 3 runs.  Returns
     (seconds, runs) for the whole path (dequantize W to f32, f32 GEMV, bias, cast) and the same for the
@@ -667,6 +704,8 @@ def main():
                     help="run only the Q4_K prefill workload (C5 at 256 rows) and print its line; for profiling")
     ap.add_argument("--read-calibration", action="store_true",
                     help="only time an empty launch and read-only passes over the rotated weight copies next to the GEMV")
+    ap.add_argument("--issue-calibration", action="store_true",
+                    help="time a wavefront's MFMAs, packed vector instructions and LDS fragment reads alone and mixed, and print the table")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 20 device-to-device copies of 256 MiB (reference dispatches for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -690,6 +729,10 @@ def main():
         return 0
     from oracle import oracle as O
     r = Runner()
+    if args.issue_calibration:
+        print(json.dumps(issue_calibration(r)))
+        return 0
+
     if args.read_calibration:
         print(json.dumps(read_calibration(r, O, min(args.steps, 2000), min(args.warmup, 100))))
         return 0

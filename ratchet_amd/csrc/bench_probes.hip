@@ -1,5 +1,6 @@
-// Measurement probes for bench.py --read-calibration: what one launch costs when it does
-// nothing, and when it only reads a buffer the size of the headline weight.  They give the
+// Measurement probes for bench.py --read-calibration and --issue-calibration: what one launch costs when it does
+// nothing, and when it only reads a buffer the size of the headline weight; and what a wavefront's MFMAs, packed
+// vector instructions and LDS fragment reads cost alone and mixed.  They give the
 // streaming kernels' times their context (how much of a launch is fixed, how fast this chip
 // delivers 27.9 MB to a kernel that has nothing else to do).  Built into their own library,
 // libratchet_probes.so; the product library does not contain them and nothing else uses them.
@@ -50,7 +51,70 @@ __global__ __launch_bounds__(1024) void probe_read_rows16_kernel(const uint8_t *
     if (acc == 0x12345678u) sink[blockIdx.x & 1023] = acc;
 }
 
+// One wavefront per SIMD (256 threads, 256 workgroups) runs `iters` trips of: NM MFMAs (16x16x32 f16, eight
+// independent accumulators), NV packed f16 FMAs behind each of eight slots, ND 16-byte-per-lane LDS reads in the
+// fragment pattern of the tiled kernels (16 rows 528 bytes apart, four lane groups 128 bytes apart), whose data
+// feed the next trip's MFMAs.  The order inside a trip is pinned: read, MFMA, vector instructions.
+typedef _Float16 probe_h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 probe_h8 __attribute__((ext_vector_type(8)));
+typedef float probe_f4 __attribute__((ext_vector_type(4)));
+template <int NV, int NM, int ND>
+__global__ __launch_bounds__(256) void probe_issue_mix_kernel(const probe_h8 *in, float *out, int iters) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    for (int i = threadIdx.x; i < 16384; i += 256) ((uint32_t *)smem)[i] = 0;
+    __syncthreads();
+    probe_h8 a = in[threadIdx.x], b = in[threadIdx.x + 256];
+    probe_f4 acc[8];
+    for (int i = 0; i < 8; i++) acc[i] = probe_f4{0, 0, 0, 0};
+    probe_h2 v[8];
+    for (int i = 0; i < 8; i++) v[i] = probe_h2{a[i], b[i]};
+    const probe_h2 m = {b[0], b[1]}, c = {b[2], b[3]};
+    const uint32_t la = (threadIdx.x & 15) * 528 + ((threadIdx.x >> 4) & 3) * 128 + (threadIdx.x >> 6) * 8448;
+    probe_h8 x[2][4];
+    for (int d = 0; d < 4; d++) x[0][d] = a, x[1][d] = b;
+    for (int it = 0; it < iters; it += 2) {
+#pragma unroll
+        for (int ph = 0; ph < 2; ph++) {
+#pragma unroll
+            for (int d = 0; d < ND; d++) x[ph ^ 1][d & 3] = __builtin_bit_cast(probe_h8, *(const probe_u4 *)(smem + la + 16 * d + 128 * ph));
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                if (i < NM) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x[ph][i & 3], b, acc[i], 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < NV; j++) v[(i + j) & 7] = __builtin_elementwise_fma(v[(i + j) & 7], m, c);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                if (ND >= 8 || (ND == 4 && (i & 1) == 0) || (ND == 2 && (i & 3) == 0)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (i < NM) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (NV) __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    float s = 0;
+    for (int i = 0; i < 8; i++) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3] + (float)v[i][0] + (float)v[i][1];
+    out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
 extern "C" {
+
+// `in`: 8 KiB of zeros; `out`: 256 KiB.  Returns hipErrorInvalidValue for a mix that is not instantiated.
+__attribute__((visibility("default"))) int probe_issue_mix(int nv, int nm, int nd, int iters, const void *in, void *out, void *stream) {
+#define PROBE_MIX(V, M, D)                                                                                                          \
+    if (nv == V && nm == M && nd == D) {                                                                                            \
+        static const hipError_t e = hipFuncSetAttribute((const void *)probe_issue_mix_kernel<V, M, D>,                              \
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 65536);                         \
+        if (e != hipSuccess) return (int)e;                                                                                         \
+        hipLaunchKernelGGL((probe_issue_mix_kernel<V, M, D>), dim3(256), dim3(256), 65536, (hipStream_t)stream,                     \
+                           (const probe_h8 *)in, (float *)out, iters);                                                             \
+        return (int)hipGetLastError();                                                                                              \
+    }
+    PROBE_MIX(0, 8, 0) PROBE_MIX(3, 0, 0) PROBE_MIX(3, 8, 0) PROBE_MIX(0, 8, 4) PROBE_MIX(3, 0, 4) PROBE_MIX(3, 8, 2) PROBE_MIX(3, 8, 4)
+    PROBE_MIX(1, 8, 0) PROBE_MIX(2, 8, 0) PROBE_MIX(4, 8, 0) PROBE_MIX(6, 8, 0)
+#undef PROBE_MIX
+    return (int)hipErrorInvalidValue;
+}
 
 __attribute__((visibility("default"))) int probe_empty(void *sink, void *stream) {
     hipLaunchKernelGGL(probe_empty_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (uint32_t *)sink);
