@@ -636,18 +636,22 @@ def issue_calibration(r: Runner):
     torch = r.torch
     P = ctypes.CDLL(os.path.join(ROOT, "ratchet_amd", "libratchet_probes.so"))
     vp = ctypes.c_void_p
-    P.probe_issue_mix.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+    P.probe_issue_mix.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
     src = torch.zeros(8192, dtype=torch.uint8, device="cuda:0")
     dst = torch.zeros(256 * 1024, dtype=torch.uint8, device="cuda:0")
     iters, rows = 4000, []
-    mixes = [("8 MFMAs", 0, 8, 0), ("24 packed FMAs", 3, 0, 0), ("8 MFMAs + 8 packed FMAs", 1, 8, 0),
-             ("8 MFMAs + 16 packed FMAs", 2, 8, 0), ("8 MFMAs + 24 packed FMAs", 3, 8, 0),
-             ("8 MFMAs + 32 packed FMAs", 4, 8, 0), ("8 MFMAs + 48 packed FMAs", 6, 8, 0),
-             ("8 MFMAs + 4 fragment reads", 0, 8, 4), ("24 packed FMAs + 4 fragment reads", 3, 0, 4),
-             ("8 MFMAs + 24 packed FMAs + 2 fragment reads", 3, 8, 2), ("8 MFMAs + 24 packed FMAs + 4 fragment reads", 3, 8, 4)]
-    for name, nv, nm, nd in mixes:
+    mixes = [("8 MFMAs", 0, 8, 0, 0), ("24 packed FMAs", 3, 0, 0, 0), ("8 MFMAs + 8 packed FMAs", 1, 8, 0, 0),
+             ("8 MFMAs + 16 packed FMAs", 2, 8, 0, 0), ("8 MFMAs + 24 packed FMAs", 3, 8, 0, 0),
+             ("8 MFMAs + 32 packed FMAs", 4, 8, 0, 0), ("8 MFMAs + 48 packed FMAs", 6, 8, 0, 0),
+             ("8 MFMAs + 4 fragment reads", 0, 8, 4, 0), ("24 packed FMAs + 4 fragment reads", 3, 0, 4, 0),
+             ("8 MFMAs + 24 packed FMAs + 2 fragment reads, each in front of an MFMA", 3, 8, 2, 0),
+             ("8 MFMAs + 24 packed FMAs + 4 fragment reads, each in front of an MFMA", 3, 8, 4, 0),
+             ("8 MFMAs + 24 packed FMAs + 8 fragment reads, each in front of an MFMA", 3, 8, 8, 0),
+             ("8 MFMAs + 24 packed FMAs + 4 fragment reads, each right behind an MFMA", 3, 8, 4, 1),
+             ("8 MFMAs + 24 packed FMAs + 8 fragment reads, each right behind an MFMA", 3, 8, 8, 1)]
+    for name, nv, nm, nd, behind in mixes:
         def launch():
-            rc = P.probe_issue_mix(nv, nm, nd, iters, vp(src.data_ptr()), vp(dst.data_ptr()), vp(torch.cuda.current_stream().cuda_stream))
+            rc = P.probe_issue_mix(nv, nm, nd, behind, iters, vp(src.data_ptr()), vp(dst.data_ptr()), vp(torch.cuda.current_stream().cuda_stream))
             if rc != 0:
                 raise RuntimeError(f"probe launch failed: hipError {rc}")
         launch()

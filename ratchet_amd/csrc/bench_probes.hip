@@ -54,11 +54,12 @@ __global__ __launch_bounds__(1024) void probe_read_rows16_kernel(const uint8_t *
 // One wavefront per SIMD (256 threads, 256 workgroups) runs `iters` trips of: NM MFMAs (16x16x32 f16, eight
 // independent accumulators), NV packed f16 FMAs behind each of eight slots, ND 16-byte-per-lane LDS reads in the
 // fragment pattern of the tiled kernels (16 rows 528 bytes apart, four lane groups 128 bytes apart), whose data
-// feed the next trip's MFMAs.  The order inside a trip is pinned: read, MFMA, vector instructions.
+// feed the next trip's MFMAs.  The order inside a trip is pinned: with PL = 0 a read goes in front of an MFMA
+// (read, MFMA, vector instructions), with PL = 1 right behind it (MFMA, read, vector instructions).
 typedef _Float16 probe_h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 probe_h8 __attribute__((ext_vector_type(8)));
 typedef float probe_f4 __attribute__((ext_vector_type(4)));
-template <int NV, int NM, int ND>
+template <int NV, int NM, int ND, int PL>
 __global__ __launch_bounds__(256) void probe_issue_mix_kernel(const probe_h8 *in, float *out, int iters) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     for (int i = threadIdx.x; i < 16384; i += 256) ((uint32_t *)smem)[i] = 0;
@@ -85,8 +86,10 @@ __global__ __launch_bounds__(256) void probe_issue_mix_kernel(const probe_h8 *in
             }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                if (ND >= 8 || (ND == 4 && (i & 1) == 0) || (ND == 2 && (i & 3) == 0)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                const bool rd = ND >= 8 || (ND == 4 && (i & 1) == 0) || (ND == 2 && (i & 3) == 0);
+                if (PL == 0 && rd) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 if (i < NM) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (PL == 1 && rd) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 if (NV) __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -100,18 +103,19 @@ __global__ __launch_bounds__(256) void probe_issue_mix_kernel(const probe_h8 *in
 extern "C" {
 
 // `in`: 8 KiB of zeros; `out`: 256 KiB.  Returns hipErrorInvalidValue for a mix that is not instantiated.
-__attribute__((visibility("default"))) int probe_issue_mix(int nv, int nm, int nd, int iters, const void *in, void *out, void *stream) {
-#define PROBE_MIX(V, M, D)                                                                                                          \
-    if (nv == V && nm == M && nd == D) {                                                                                            \
-        static const hipError_t e = hipFuncSetAttribute((const void *)probe_issue_mix_kernel<V, M, D>,                              \
+__attribute__((visibility("default"))) int probe_issue_mix(int nv, int nm, int nd, int behind, int iters, const void *in, void *out, void *stream) {
+#define PROBE_MIX(V, M, D, P)                                                                                                       \
+    if (nv == V && nm == M && nd == D && behind == P) {                                                                                          \
+        static const hipError_t e = hipFuncSetAttribute((const void *)probe_issue_mix_kernel<V, M, D, P>,                              \
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 65536);                         \
         if (e != hipSuccess) return (int)e;                                                                                         \
-        hipLaunchKernelGGL((probe_issue_mix_kernel<V, M, D>), dim3(256), dim3(256), 65536, (hipStream_t)stream,                     \
+        hipLaunchKernelGGL((probe_issue_mix_kernel<V, M, D, P>), dim3(256), dim3(256), 65536, (hipStream_t)stream,                     \
                            (const probe_h8 *)in, (float *)out, iters);                                                             \
         return (int)hipGetLastError();                                                                                              \
     }
-    PROBE_MIX(0, 8, 0) PROBE_MIX(3, 0, 0) PROBE_MIX(3, 8, 0) PROBE_MIX(0, 8, 4) PROBE_MIX(3, 0, 4) PROBE_MIX(3, 8, 2) PROBE_MIX(3, 8, 4)
-    PROBE_MIX(1, 8, 0) PROBE_MIX(2, 8, 0) PROBE_MIX(4, 8, 0) PROBE_MIX(6, 8, 0)
+    PROBE_MIX(0, 8, 0, 0) PROBE_MIX(3, 0, 0, 0) PROBE_MIX(3, 8, 0, 0) PROBE_MIX(0, 8, 4, 0) PROBE_MIX(3, 0, 4, 0) PROBE_MIX(3, 8, 2, 0)
+    PROBE_MIX(3, 8, 4, 0) PROBE_MIX(1, 8, 0, 0) PROBE_MIX(2, 8, 0, 0) PROBE_MIX(4, 8, 0, 0) PROBE_MIX(6, 8, 0, 0)
+    PROBE_MIX(3, 8, 4, 1) PROBE_MIX(3, 8, 8, 0) PROBE_MIX(3, 8, 8, 1)
 #undef PROBE_MIX
     return (int)hipErrorInvalidValue;
 }

@@ -264,8 +264,11 @@ __global__ __launch_bounds__(64 * (MW + QR_LW)) void gemm_q4k_kernel(GemmQ4kArgs
         };
         half8_t xf[2][TB];
         xread(0, xf[0]);
-        // The order inside a super-block is the compiler's: pinning the fragment reads a step ahead of their MFMAs, or
-        // spreading them one per two MFMAs, measured the same or slower.
+        // The order inside a super-block is the compiler's.  Pinned orders were measured: fragment reads a step ahead
+        // of their MFMAs, one read in front of every second MFMA, one right behind every MFMA (where a bare loop of
+        // MFMAs, packed FMAs and fragment reads issues them for 2 ns instead of 10: bench.py --issue-calibration);
+        // with two weight tiles per wavefront all were the same or up to 4 % slower, with one tile the last was
+        // 6 % faster.
         auto mfma_step = [&](auto Tc) {
             constexpr int T = decltype(Tc)::value;
             if constexpr (T < 7) xread(T + 1, xf[(T + 1) & 1]);
