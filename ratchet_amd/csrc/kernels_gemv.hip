@@ -323,7 +323,7 @@ hipError_t launch_gemv(const Problem &p, const void *A, const void *B, const voi
         e = launch_gemv_q4k_mfma(p, A, B, bias, out, stream, dev);
         if (e != hipErrorNotSupported) return e;
     }
-    if (p.kernel == RT_KERNEL_GEMV_FLOAT) { // one vector, rows of whole 16-byte vectors up to 10 KiB: the row-streaming kernel
+    if (p.kernel == RT_KERNEL_GEMV_FLOAT) { // up to four vectors, rows of whole 16-byte vectors: the row-streaming kernel
         hipError_t e = launch_gemv_float_rowdot(p, A, B, bias, out, stream, dev);
         if (e != hipErrorNotSupported) return e;
     }

@@ -1,5 +1,5 @@
 // Row-streaming GEMV for f16 and f32 weights, one activation vector (the decode step of an
-// unquantized checkpoint).
+// unquantized checkpoint) or a few.
 //
 //   y[n] = sum_k W[n, k] * x[k]  (+ bias)
 //
@@ -29,18 +29,24 @@ struct GemvRowFloatArgs {
     uint8_t *out;
     uint32_t M;             // weight rows
     uint32_t nvec;          // 16-byte vectors per row
-    uint32_t bias_rs;       // 1: a bias per weight row, 0: one for the vector
+    uint32_t bias_rs;       // 1: a bias per weight row, 0: one per activation vector
+    uint32_t bias_js;       // 1: a bias per activation vector, 0: one per weight row (or none)
+    uint32_t NC;            // activation vectors (1 .. the kernel's NCT)
     int64_t a_rs;           // bytes between rows
-    int64_t o_is;           // elements between the outputs of consecutive rows
+    int64_t x_js;           // bytes between activation vectors
+    int64_t o_is, o_js;     // elements between the outputs of consecutive rows / vectors
     int64_t a_ss, x_ss, o_ss; // per stack: bytes of weights, bytes of activations, output elements
     int has_bias, act;
 };
 
-template <typename AT, int STEPS, int WAVES>
+// NCT: activation vectors the kernel is built for (1, 2, 4); with fewer (g.NC) the spare ones repeat the last and are
+// not stored.  The weights are read once for all of them; every vector adds its staged copy, its registers and its
+// dot products.
+template <typename AT, int STEPS, int WAVES, int NCT>
 __global__ __launch_bounds__(WAVES * 64) void gemv_float_rowdot_kernel(GemvRowFloatArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int THREADS = WAVES * 64;
-    uint4_t *xs = (uint4_t *)smem; // [nvec]
+    uint4_t *xs = (uint4_t *)smem; // [NCT][nvec]
     const int t = threadIdx.x, lane = t & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t nwg = gridDim.x;
@@ -58,13 +64,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_float_rowdot_kernel(GemvRowFl
     }
     const uint32_t nvec = g.nvec;
 
-    // 1. the activations: the workgroup stages the whole vector
+    // 1. the activations: the workgroup stages the whole vectors
     constexpr int XV = (64 * STEPS + THREADS - 1) / THREADS;
-    uint4_t xv[XV];
+    uint4_t xv[NCT][XV];
 #pragma unroll
-    for (int i = 0; i < XV; i++) {
-        const uint32_t v = min((uint32_t)(i * THREADS + t), nvec - 1); // threads past the end re-read the last vector
-        xv[i] = *(const uint4_t *)(xg + 16 * v);
+    for (int j = 0; j < NCT; j++) {
+        const uint8_t *xj = NCT == 1 ? xg : xg + (int64_t)min((uint32_t)j, g.NC - 1) * g.x_js;
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const uint32_t v = min((uint32_t)(i * THREADS + t), nvec - 1); // threads past the end re-read the last vector
+            xv[j][i] = *(const uint4_t *)(xj + 16 * v);
+        }
     }
     asm volatile("" ::: "memory"); // keep the loads in this order
     // 2. the row: 16 bytes per lane and step; only the last step can be short, its spare lanes re-read the row's end
@@ -75,45 +85,63 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_float_rowdot_kernel(GemvRowFl
     w[STEPS - 1] = __builtin_nontemporal_load((const uint4_t *)(abase + 16 * vl));
     asm volatile("" ::: "memory");
     // 3. the epilogue's bias, unconditional (a branch here would wait for every load above)
-    const AT braw = *(const AT *)(g.bias + sizeof(AT) * (size_t)((row0 + rc) * g.bias_rs));
+    AT braw[NCT];
+#pragma unroll
+    for (int j = 0; j < NCT; j++)
+        braw[j] = *(const AT *)(g.bias + sizeof(AT) * (size_t)((row0 + rc) * g.bias_rs + min((uint32_t)j, g.NC - 1) * g.bias_js));
     asm volatile("" ::: "memory");
     // where this row goes: computed while the loads are on their way
     AT *op = obase + (int64_t)(row0 + wave) * g.o_is;
     asm volatile("" : "+v"(op));
     // 4. activations -> LDS; the barrier waits for the LDS writes, not for the weights
 #pragma unroll
-    for (int i = 0; i < XV; i++) {
-        const uint32_t v = i * THREADS + t;
-        if (v < nvec) xs[v] = xv[i];
-    }
+    for (int j = 0; j < NCT; j++)
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const uint32_t v = i * THREADS + t;
+            if (v < nvec) xs[j * nvec + v] = xv[j][i];
+        }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0); // nothing that touches a weight moves above the barrier or between the LDS reads
-    uint4_t xr[STEPS];
+    uint4_t xr[NCT][STEPS];
 #pragma unroll
-    for (int st = 0; st < STEPS - 1; st++) xr[st] = xs[64 * st + lane];
-    xr[STEPS - 1] = xs[vl];
+    for (int j = 0; j < NCT; j++) {
+#pragma unroll
+        for (int st = 0; st < STEPS - 1; st++) xr[j][st] = xs[j * nvec + 64 * st + lane];
+        xr[j][STEPS - 1] = xs[j * nvec + vl];
+    }
     __builtin_amdgcn_sched_barrier(0);
     // 5. dot products
-    float acc = 0.f;
+    float acc[NCT];
+#pragma unroll
+    for (int j = 0; j < NCT; j++) acc[j] = 0.f;
 #pragma unroll
     for (int st = 0; st < STEPS; st++) {
-        float p = 0.f;
+        const bool spare = st == STEPS - 1 && (uint32_t)(64 * (STEPS - 1) + lane) >= nvec; // a spare lane of the short step
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-            const uint32_t ww = w[st][d], xw = xr[st][d];
-            if constexpr (sizeof(AT) == 2) p = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ww), __builtin_bit_cast(half2_t, xw), p, false);
-            else p = fmaf(__builtin_bit_cast(float, ww), __builtin_bit_cast(float, xw), p);
+        for (int j = 0; j < NCT; j++) {
+            float p = 0.f;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t ww = w[st][d], xw = xr[j][st][d];
+                if constexpr (sizeof(AT) == 2) p = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ww), __builtin_bit_cast(half2_t, xw), p, false);
+                else p = fmaf(__builtin_bit_cast(float, ww), __builtin_bit_cast(float, xw), p);
+            }
+            acc[j] += spare ? 0.f : p;
         }
-        if (st == STEPS - 1 && (uint32_t)(64 * (STEPS - 1) + lane) >= nvec) p = 0.f; // a spare lane of the short step
-        acc += p;
     }
     // 6. the row's lanes meet; one lane writes
-    const float v = rowdot_sum<true>(acc);
+    float v[NCT];
+#pragma unroll
+    for (int j = 0; j < NCT; j++) v[j] = rowdot_sum<true>(acc[j]);
     if (lane == 63 && wave <= last) {
-        const float b = g.has_bias ? to_f32(braw) : 0.f;
-        *op = from_f32<AT>(rt_act(v + b, g.act));
+#pragma unroll
+        for (int j = 0; j < NCT; j++) {
+            const float b = g.has_bias ? to_f32(braw[j]) : 0.f;
+            if (NCT == 1 || (uint32_t)j < g.NC) op[j * g.o_js] = from_f32<AT>(rt_act(v[j] + b, g.act));
+        }
     }
 }
 
@@ -210,36 +238,42 @@ RT_TUNABLE(g_gemv_rowfloat_disable, 0);
 // Tunable: wavefronts (= rows) per workgroup, 0 = by the size of the grid.
 RT_TUNABLE(g_gemv_rowfloat_waves, 0);
 
-template <typename AT, int STEPS, int WAVES>
+template <typename AT, int STEPS, int WAVES, int NCT>
 static hipError_t launch_rowfloat_w(dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
-    hipLaunchKernelGGL((gemv_float_rowdot_kernel<AT, STEPS, WAVES>), grid, dim3(WAVES * 64), lds, st, g);
+    hipLaunchKernelGGL((gemv_float_rowdot_kernel<AT, STEPS, WAVES, NCT>), grid, dim3(WAVES * 64), lds, st, g);
     return hipGetLastError();
 }
 
+// nct: 1, 2 or 4 vectors; more than one only with four wavefronts per workgroup, four only for f16 rows of up to 5 KiB
 template <typename AT, int STEPS>
-static hipError_t launch_rowfloat(int waves, dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
-    if (waves == 4) return launch_rowfloat_w<AT, STEPS, 4>(grid, lds, st, g);
+static hipError_t launch_rowfloat(int waves, int nct, dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
+    if (nct == 2) return launch_rowfloat_w<AT, STEPS, 4, 2>(grid, lds, st, g);
+    if constexpr (sizeof(AT) == 2 && STEPS <= 5) {
+        if (nct == 4) return launch_rowfloat_w<AT, STEPS, 4, 4>(grid, lds, st, g);
+    }
+    if (nct != 1) return hipErrorNotSupported;
+    if (waves == 4) return launch_rowfloat_w<AT, STEPS, 4, 1>(grid, lds, st, g);
 #ifdef RT_DEV_TUNABLES
-    if (waves == 8) return launch_rowfloat_w<AT, STEPS, 8>(grid, lds, st, g);
-    if (waves == 5) return launch_rowfloat_w<AT, STEPS, 5>(grid, lds, st, g);
-    if (waves == 10) return launch_rowfloat_w<AT, STEPS, 10>(grid, lds, st, g);
+    if (waves == 8) return launch_rowfloat_w<AT, STEPS, 8, 1>(grid, lds, st, g);
+    if (waves == 5) return launch_rowfloat_w<AT, STEPS, 5, 1>(grid, lds, st, g);
+    if (waves == 10) return launch_rowfloat_w<AT, STEPS, 10, 1>(grid, lds, st, g);
 #endif
-    return launch_rowfloat_w<AT, STEPS, 2>(grid, lds, st, g);
+    return launch_rowfloat_w<AT, STEPS, 2, 1>(grid, lds, st, g);
 }
 
 template <typename AT>
-static hipError_t launch_rowfloat_steps(int steps, int waves, dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
+static hipError_t launch_rowfloat_steps(int steps, int waves, int nct, dim3 grid, size_t lds, hipStream_t st, const GemvRowFloatArgs &g) {
     switch (steps) {
-    case 1: return launch_rowfloat<AT, 1>(waves, grid, lds, st, g);
-    case 2: return launch_rowfloat<AT, 2>(waves, grid, lds, st, g);
-    case 3: return launch_rowfloat<AT, 3>(waves, grid, lds, st, g);
-    case 4: return launch_rowfloat<AT, 4>(waves, grid, lds, st, g);
-    case 5: return launch_rowfloat<AT, 5>(waves, grid, lds, st, g);
-    case 6: return launch_rowfloat<AT, 6>(waves, grid, lds, st, g);
-    case 7: return launch_rowfloat<AT, 7>(waves, grid, lds, st, g);
-    case 8: return launch_rowfloat<AT, 8>(waves, grid, lds, st, g);
-    case 9: return launch_rowfloat<AT, 9>(waves, grid, lds, st, g);
-    case 10: return launch_rowfloat<AT, 10>(waves, grid, lds, st, g);
+    case 1: return launch_rowfloat<AT, 1>(waves, nct, grid, lds, st, g);
+    case 2: return launch_rowfloat<AT, 2>(waves, nct, grid, lds, st, g);
+    case 3: return launch_rowfloat<AT, 3>(waves, nct, grid, lds, st, g);
+    case 4: return launch_rowfloat<AT, 4>(waves, nct, grid, lds, st, g);
+    case 5: return launch_rowfloat<AT, 5>(waves, nct, grid, lds, st, g);
+    case 6: return launch_rowfloat<AT, 6>(waves, nct, grid, lds, st, g);
+    case 7: return launch_rowfloat<AT, 7>(waves, nct, grid, lds, st, g);
+    case 8: return launch_rowfloat<AT, 8>(waves, nct, grid, lds, st, g);
+    case 9: return launch_rowfloat<AT, 9>(waves, nct, grid, lds, st, g);
+    case 10: return launch_rowfloat<AT, 10>(waves, nct, grid, lds, st, g);
     default: return hipErrorNotSupported;
     }
 }
@@ -264,12 +298,14 @@ static hipError_t launch_rowlong(bool f16, int waves, dim3 grid, size_t lds, hip
     return waves == 4 ? launch_rowlong_w<float, 4>(grid, lds, st, g) : launch_rowlong_w<float, 2>(grid, lds, st, g);
 }
 
-// f16 or f32 weights with rows of whole 16-byte vectors, at most 64 KiB long, one activation vector of the same type.
+// f16 or f32 weights with rows of whole 16-byte vectors, at most 64 KiB long, one activation vector of the same type;
+// rows of up to 10 KiB also two vectors, f16 rows of up to 5 KiB up to four (10240 x 2560 f16: 2 / 4 vectors 11.0 / 14
+// us on the one-load-at-a-time kernel).
 // hipErrorNotSupported: the shape or alignment does not fit and another kernel must run.
 hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                     hipStream_t stream, const DeviceInfo &dev) {
     if (g_gemv_rowfloat_disable) return hipErrorNotSupported;
-    if (p.kernel != RT_KERNEL_GEMV_FLOAT || (p.act_dt != RT_F16 && p.act_dt != RT_F32) || p.N != 1) return hipErrorNotSupported;
+    if (p.kernel != RT_KERNEL_GEMV_FLOAT || (p.act_dt != RT_F16 && p.act_dt != RT_F32) || p.N < 1 || p.N > 4) return hipErrorNotSupported;
     if (p.stacks > 65535 || p.a_ks != 1 || p.b_ks != 1 || p.M < 1 || p.M > 0x7fffffff) return hipErrorNotSupported;
     const int64_t esz = p.act_dt == RT_F16 ? 2 : 4;
     const int64_t row_bytes = p.K * esz;
@@ -278,10 +314,14 @@ hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void 
         return hipErrorNotSupported;
     const uint32_t nvec = (uint32_t)(row_bytes / 16);
     const int steps = (int)((nvec + 63) / 64);
+    const int nct = p.N == 1 ? 1 : p.N == 2 ? 2 : 4;
+    if (nct > 1 && (steps > 10 || (p.b_js * esz) % 16 != 0)) return hipErrorNotSupported;
+    if (nct == 4 && (p.act_dt != RT_F16 || steps > 5)) return hipErrorNotSupported;
     // four rows per workgroup; two where that leaves the grid under three workgroups per compute unit
     int waves = 4;
     if ((p.M + 3) / 4 * p.stacks < 3 * (int64_t)dev.num_cus) waves = 2;
     if (g_gemv_rowfloat_waves > 0) waves = g_gemv_rowfloat_waves;
+    if (nct > 1) waves = 4;
     const int64_t groups = (p.M + waves - 1) / waves;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
 
@@ -289,16 +329,20 @@ hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void 
     g.A = (const uint8_t *)A, g.X = (const uint8_t *)B, g.out = (uint8_t *)out;
     g.bias = p.has_bias ? (const uint8_t *)bias : (const uint8_t *)B;
     g.bias_rs = p.has_bias && p.bias_on_rows ? 1u : 0u;
+    g.bias_js = p.has_bias && !p.bias_on_rows ? 1u : 0u;
+    g.NC = (uint32_t)p.N;
+    g.x_js = p.N == 1 ? 0 : p.b_js * esz;
+    g.o_js = p.o_js;
     g.M = (uint32_t)p.M, g.nvec = nvec;
     g.a_rs = p.a_rs * esz;
     g.o_is = p.o_is;
     g.a_ss = p.a_stack == 1 ? 0 : p.a_bs * esz, g.x_ss = p.b_stack == 1 ? 0 : p.b_bs * esz, g.o_ss = p.o_bs;
     g.has_bias = p.has_bias, g.act = p.act;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
-    const size_t lds = (size_t)nvec * 16;
+    const size_t lds = (size_t)nct * nvec * 16;
     if (steps > 10) return launch_rowlong(p.act_dt == RT_F16, waves, grid, lds, stream, g);
-    return p.act_dt == RT_F16 ? launch_rowfloat_steps<half_t>(steps, waves, grid, lds, stream, g)
-                              : launch_rowfloat_steps<float>(steps, waves, grid, lds, stream, g);
+    return p.act_dt == RT_F16 ? launch_rowfloat_steps<half_t>(steps, waves, nct, grid, lds, stream, g)
+                              : launch_rowfloat_steps<float>(steps, waves, nct, grid, lds, stream, g);
 }
 
 } // namespace rt

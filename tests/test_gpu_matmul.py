@@ -494,6 +494,42 @@ def test_float_gemv_paths(device, oracle, dt):
 
 
 @pytest.mark.parametrize("dt", [DType.F32, DType.F16], ids=["f32", "f16"])
+def test_float_row_streaming_few_vectors(device, oracle, dt):
+    """f16 / f32 weights against two activation vectors (rows of up to 10 KiB), and f16 against three or four
+    (rows of up to 5 KiB), take the row-streaming kernel too: step counts, short last steps, stacks with
+    broadcast, a bias along the weight rows or along the vectors, both output orientations, a fused activation.
+    Other counts and longer rows fall to the one-load-at-a-time kernel and must agree as well."""
+    npdt = dt.numpy()
+    E = 16 // np.dtype(npdt).itemsize
+    cases = [(1, 70, 64 * E * k, 2) for k in (1, 2, 5, 7, 10)] + [(1, 33, E, 2), (1, 1030, 65 * E, 2), (2, 19, 96 * E, 2),
+             (1, 10240, 2560, 2), (1, 41, 64 * E * 3 + 3 * E, 3), (1, 77, 64 * E * 5, 4), (1, 10240, 2560, 4), (2, 9, 300 * E, 4),
+             (1, 50, 64 * E * 6, 4), (1, 50, 64 * E * 2, 5), (1, 37, 641 * E, 2)]
+    for i, (S, N, K, M) in enumerate(cases):
+        rng = np.random.default_rng(560 + i)
+        for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
+            w = rng.standard_normal((ws, N, K)).astype(npdt)
+            x = rng.standard_normal((xs_, M, K)).astype(npdt)
+            for to in (True, False):
+                bias = rng.standard_normal(N if to else M).astype(npdt) if (i + to) % 3 else None
+                got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x),
+                                 None if bias is None else Tensor.from_data(bias), False, True, to)
+                want = oracle.matmul_ref(w, int(dt), w.shape, x, int(dt), x.shape, bias, False, True, to)
+                check(oracle, got, want, dt, (S, ws, xs_, N, K, M, to))
+    rng = np.random.default_rng(580)
+    N, K, M = 100, 1536, 3
+    w, x, bias = (rng.standard_normal(sh).astype(npdt) for sh in ((N, K), (1, M, K), (N,)))
+    y = Tensor.from_data(w).to(device).gemm(Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device), False, True, True).gelu().resolve()
+    want = oracle.matmul_ref(w, int(dt), w.shape, x, int(dt), x.shape, bias, False, True, True, act=oracle.ACT_GELU)
+    assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
+    # one-hot activations return weight columns bit for bit
+    cols = rng.integers(0, K, size=M)
+    x1 = np.zeros((1, M, K), dtype=npdt)
+    x1[0, np.arange(M), cols] = 1
+    got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x1), None, False, True, True)
+    assert np.array_equal(got[0], w[:, cols].T)
+
+
+@pytest.mark.parametrize("dt", [DType.F32, DType.F16], ids=["f32", "f16"])
 def test_float_row_streaming_one_vector(device, oracle, dt):
     """f16 / f32 weights against one vector take the row-streaming kernels while a row is whole 16-byte vectors
     and at most 64 KiB: every step count (1..10 KiB of row), rows whose last step is short or a single
