@@ -75,7 +75,9 @@ __device__ __forceinline__ half8_t q4k_scaled(uint32_t v0, uint32_t v1, half_t s
 // wavefronts per SIMD run the same instructions at the same time), so that shows.
 // RG: 16-row groups per workgroup (1 or 2).  They share the staged activations; with 9..16 vectors those leave room
 // for one workgroup per compute unit, and two row groups then cover 8192 rows in one round of 256 workgroups.
-template <int NCT, bool FAST, int RG>
+// SBW: super-blocks per wavefront (1, or 2 for K above 4096: wavefront w takes super-blocks w and w + nwaves, all of
+// whose loads are issued before the first is consumed).
+template <int NCT, bool FAST, int RG, int SBW>
 __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int XROW = 256 + kQ4kXPad; // halfs per staged activation row (one super-block of K)
@@ -94,14 +96,18 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     const uint32_t nwg = gridDim.x;
     const uint32_t wg = (nwg & 7) == 0 ? (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3) : blockIdx.x;
     const int64_t row0 = (int64_t)wg * (FAST ? 16 * RG : g.rows_wg);
-    const bool live = FAST || wave < g.nsb; // padding waves (nwaves > nsb) contribute zero
-    const int sbi = live ? wave : 0;
-
-    // 1. this wave's 256 activations per vector: 32 16-byte vectors per row
+    // 1. this wave's 256 activations per vector and super-block: 32 16-byte vectors per row
     constexpr int XL = (NCT * 32 + 63) / 64;
     const int nvec = NC * 32;
-    uint4_t xv[XL], hdr_[RG], qa_[RG], qb_[RG];
+    uint4_t xv_[SBW][XL], hdr__[SBW][RG], qa__[SBW][RG], qb__[SBW][RG];
     uint32_t bias_raw_[RG];
+    bool live_[SBW];
+#pragma unroll
+    for (int pass = 0; pass < SBW; pass++) {
+    uint4_t (&xv)[XL] = xv_[pass], (&hdr_)[RG] = hdr__[pass], (&qa_)[RG] = qa__[pass], (&qb_)[RG] = qb__[pass];
+    const bool live = FAST || wave + pass * nwaves < g.nsb; // padding waves (nwaves * SBW > nsb) contribute zero
+    live_[pass] = live;
+    const int sbi = live ? wave + pass * nwaves : 0;
     if constexpr (FAST) {
         const half_t *xg = g.X + sbi * 256;
 #pragma unroll
@@ -156,6 +162,11 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
         asm volatile("" ::: "memory");
     }
 
+    }
+#pragma unroll
+    for (int pass = 0; pass < SBW; pass++) {
+    const uint4_t (&xv)[XL] = xv_[pass], (&hdr_)[RG] = hdr__[pass], (&qa_)[RG] = qa__[pass], (&qb_)[RG] = qb__[pass];
+    const bool live = live_[pass];
     // 3. activations -> LDS, and the sums of x over each sub-block of 32 as f16 high + low parts
 #pragma unroll
     for (int i = 0; i < XL; i++) {
@@ -229,8 +240,13 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
         constexpr int NR = NCT < 4 ? NCT : 4;
         if (NCT >= 16 || 4 * grp < NCT) {
 #pragma unroll
-            for (int r = 0; r < NR; r++) psum[(wave * RG + rg) * 256 + (4 * grp + r) * 16 + n] = fmaf(-dmin, T[r], d * P[r]);
+            for (int r = 0; r < NR; r++) {
+                float &ps = psum[(wave * RG + rg) * 256 + (4 * grp + r) * 16 + n];
+                ps = fmaf(-dmin, T[r], d * P[r]) + (pass == 0 ? 0.f : ps);
+            }
         }
+    }
+    if (SBW > 1) asm volatile("" ::: "memory"); // the next pass restages the activations behind this pass's reads (DS operations complete in order)
     }
 
     // 7. sum the K slices
@@ -248,21 +264,28 @@ __global__ __launch_bounds__(1024) void gemv_q4k_mfma_kernel(GemvQ4kArgs g) {
     }
 }
 
-template <int NCT, bool FAST, int RG>
+template <int NCT, bool FAST, int RG, int SBW = 1>
 static hipError_t launch_q4k_kernel(dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvQ4kArgs &g) {
     if (lds > 48 * 1024) {
-        const hipError_t e = ensure_lds_limit<&gemv_q4k_mfma_kernel<NCT, FAST, RG>>();
+        const hipError_t e = ensure_lds_limit<&gemv_q4k_mfma_kernel<NCT, FAST, RG, SBW>>();
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<NCT, FAST, RG>), grid, dim3(nwaves * 64), lds, st, g);
+    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<NCT, FAST, RG, SBW>), grid, dim3(nwaves * 64), lds, st, g);
     return hipGetLastError();
 }
 
 template <int NCT>
-static hipError_t launch_q4k_one(int rg, dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvQ4kArgs &g) {
+static hipError_t launch_q4k_one(int rg, int sbw, dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvQ4kArgs &g) {
     const bool regular = grid.y == 1 && g.a_stack == 1 && g.b_stack == 1 && g.M % (16 * rg) == 0 && g.rows_wg == 16 * rg &&
-                         g.NC == NCT && g.nsb == nwaves && g.M * g.nsb * 144 < (int64_t(1) << 31) &&
+                         g.NC == NCT && g.nsb == nwaves * sbw && g.M * g.nsb * 144 < (int64_t(1) << 31) &&
                          (int64_t)g.NC * g.b_js < (int64_t(1) << 30);
+    if constexpr (NCT <= 8) { // two super-blocks per wavefront: K above 4096
+        if (sbw == 2) {
+            if (rg != 1) return hipErrorInvalidValue;
+            return regular ? launch_q4k_kernel<NCT, true, 1, 2>(grid, nwaves, lds, st, g) : launch_q4k_kernel<NCT, false, 1, 2>(grid, nwaves, lds, st, g);
+        }
+    }
+    if (sbw != 1) return hipErrorNotSupported;
     if constexpr (NCT == 16) { // two row groups are only dealt where 9..16 vectors leave room for one workgroup per compute unit
         if (rg == 2) return regular ? launch_q4k_kernel<NCT, true, 2>(grid, nwaves, lds, st, g) : launch_q4k_kernel<NCT, false, 2>(grid, nwaves, lds, st, g);
     }
@@ -276,12 +299,12 @@ RT_TUNABLE(g_gemv_q4k_disable_mfma, 0);
 // Tunable: 1 or 2 forces that many 16-row groups per workgroup (0 = by residency, see the launcher).
 RT_TUNABLE(g_gemv_q4k_mfma_rg, 0);
 
-// Q4_K weights, f16 activations, 1..16 vectors, K a multiple of 256 and at most 4096.
+// Q4_K weights, f16 activations, 1..16 vectors, K a multiple of 256 and at most 4096 (8192 with up to 8 vectors).
 // hipErrorNotSupported means another kernel must run.
 hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                 hipStream_t stream, const DeviceInfo &dev) {
     if (g_gemv_q4k_disable_mfma) return hipErrorNotSupported;
-    if (p.a_dt != RT_Q4_K || p.act_dt != RT_F16 || p.N < 1 || p.N > 16 || p.K % 256 != 0 || p.K < 256 || p.K > 4096)
+    if (p.a_dt != RT_Q4_K || p.act_dt != RT_F16 || p.N < 1 || p.N > 16 || p.K % 256 != 0 || p.K < 256 || p.K > (p.N <= 8 ? 8192 : 4096))
         return hipErrorNotSupported;
     if (p.stacks > 65535 || p.b_ks != 1) return hipErrorNotSupported;
     const int64_t bjs = p.N == 1 ? 0 : p.b_js;
@@ -294,7 +317,8 @@ hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, 
     g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
     if (p.has_bias && ((uintptr_t)bias & 1u)) return hipErrorNotSupported;
-    const int nwaves = g.nsb < 4 ? 4 : g.nsb; // the final sum uses 256 threads
+    const int sbw = g.nsb > 16 ? 2 : 1;       // K above 4096: two super-blocks per wavefront
+    const int nwaves = g.nsb < 4 ? 4 : (g.nsb + sbw - 1) / sbw; // the final sum uses 256 threads
     // Rows per workgroup: 16, unless the activations' LDS (9..16 vectors) leaves one workgroup per compute unit and
     // the 16-row workgroups would run in rounds; then every compute unit gets one workgroup with its share of the
     // rows, up to 32 (8192 rows, 16 vectors: 512 workgroups in two rounds 9.3 us -> 256 in one 7.7 us).
@@ -311,11 +335,11 @@ hipError_t launch_gemv_q4k_mfma(const Problem &p, const void *A, const void *B, 
     const int64_t groups = (p.M + rows_wg - 1) / rows_wg;
     if (groups > 0x7fffffff) return hipErrorNotSupported;
     dim3 grid((unsigned)groups, (unsigned)p.stacks);
-    if (g.NC <= 1) return launch_q4k_one<1>(rg, grid, nwaves, lds, stream, g);
-    if (g.NC <= 2) return launch_q4k_one<2>(rg, grid, nwaves, lds, stream, g);
-    if (g.NC <= 4) return launch_q4k_one<4>(rg, grid, nwaves, lds, stream, g);
-    if (g.NC <= 8) return launch_q4k_one<8>(rg, grid, nwaves, lds, stream, g);
-    return launch_q4k_one<16>(rg, grid, nwaves, lds, stream, g);
+    if (g.NC <= 1) return launch_q4k_one<1>(rg, sbw, grid, nwaves, lds, stream, g);
+    if (g.NC <= 2) return launch_q4k_one<2>(rg, sbw, grid, nwaves, lds, stream, g);
+    if (g.NC <= 4) return launch_q4k_one<4>(rg, sbw, grid, nwaves, lds, stream, g);
+    if (g.NC <= 8) return launch_q4k_one<8>(rg, sbw, grid, nwaves, lds, stream, g);
+    return launch_q4k_one<16>(rg, sbw, grid, nwaves, lds, stream, g);
 }
 
 } // namespace rt

@@ -443,6 +443,35 @@ def test_q4k_row_streaming_long_rows(device, oracle):
             assert np.array_equal(got.reshape(-1), dq[:, col].astype(np.float16)), (N, K, col)
 
 
+def test_q4k_streaming_long_rows_few_vectors(device, oracle):
+    """Q4_K weights with K above 4096 (up to 8192) against 2..8 vectors: the matrix-core streaming kernel with two
+    super-blocks per wavefront (an odd number of super-blocks leaves the last wavefront's second one empty); row counts
+    off the 16 rows of a workgroup, stacks, both bias orientations; one-hot activations return the dequantized
+    columns bit for bit."""
+    cases = [(1, 50, 4352, 2), (1, 9, 5120, 3), (1, 16, 6144, 8), (1, 37, 8192, 5), (1, 3072, 8192, 2), (2, 21, 7168, 4),
+             (1, 130, 7936, 7)]
+    for i, (S, N, K, M) in enumerate(cases):
+        rng = np.random.default_rng(490 + i)
+        for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
+            blocks = oracle.q4k_quantize((rng.standard_normal((ws, N, K)) * 0.02).astype(np.float32))
+            x = rng.standard_normal((xs_, M, K)).astype(np.float16)
+            for to in (True, False):
+                bias = rng.standard_normal(N if to else M).astype(np.float16) if (i + to) % 3 else None
+                got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (ws, N, K)), Tensor.from_data(x),
+                                 None if bias is None else Tensor.from_data(bias), False, True, to)
+                want = oracle.matmul_ref(blocks, oracle.Q4_K, (ws, N, K), x, oracle.F16, x.shape, bias, False, True, to)
+                check(oracle, got, want, DType.F16, (S, ws, xs_, N, K, M, to))
+    rng = np.random.default_rng(499)
+    N, K, M = 23, 8192, 6
+    blocks = oracle.q4k_quantize((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    dq = oracle.q4k_dequantize(blocks).reshape(N, K)
+    cols = np.array([0, K - 1, 4095, 4096, 255, int(rng.integers(0, K))])
+    x = np.zeros((1, M, K), dtype=np.float16)
+    x[0, np.arange(M), cols] = 1
+    got = gpu_matmul(device, Tensor.from_quantized(blocks, DType.Q4_K, (N, K)), Tensor.from_data(x), None, False, True, True)
+    assert np.array_equal(got[0], dq[:, cols].T.astype(np.float16))
+
+
 def test_q4k_one_hot_is_bit_exact_dequant(device, oracle):
     rng = np.random.default_rng(401)
     N, K = 40, 512
