@@ -40,7 +40,7 @@ INFINITY_CACHE_BYTES = 256 << 20
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy); the commands and
 # readings are in profiles/gemv_q8_phi2_m1_pmc.txt.  A counter reading cannot be taken inside
 # this script, so the figure is the recorded one for the M=1 workload.
-GEMV_TRAFFIC_BYTES = 27985471
+GEMV_TRAFFIC_BYTES = 27985470
 # The same for the f16 GEMM of the metric's second half (profiles/gemm_c4_f16_q8_pmc.txt): FETCH_SIZE
 # 36,025 KiB x 1.99982 (copy calibration) + WRITE_SIZE 11,531 KiB.  The weight is read once and the
 # activations once per XCD (eight L2s), which is what puts it above the 65.6 MB the shape holds.
