@@ -25,7 +25,7 @@
 // A workgroup owns 128 weight rows x 64 activation rows: four multiplying wavefronts (32 weight rows
 // x 64 activation rows each: 64 MFMAs per super-block, 8 for the min term) and four that only issue
 // the activation tiles' LDS-DMA loads (one per SIMD, so that no multiplying wavefront shares its SIMD
-// with all of them), two super-blocks ahead in a ring of three stages.  A staged row is 32 K-vectors
+// with all of them), one super-block ahead in a ring of two stages.  A staged row is 32 K-vectors
 // and one of padding: the 16 rows of a fragment read start 4 banks apart and a read address is a
 // base + 16 * step, an immediate.  One barrier per super-block.  The output tile leaves through LDS
 // as 16-byte stores when the output is contiguous along the weight rows.
@@ -63,7 +63,10 @@ constexpr int QR_BN = 64; // activation rows per workgroup; weight rows: 16 per 
 // so that the 16 rows of a fragment read start 4 banks apart and a read address is base + 16 * step.
 constexpr int QR_ROWB = 33 * 16;       // bytes per staged row
 constexpr int QR_XSB = QR_BN * QR_ROWB; // bytes per stage = 33 LDS-DMA instructions of 1 KB
-constexpr int QR_XST = 3;              // activation stages: a tile's slots are in flight for two super-blocks
+// Activation stages: the tile of the next super-block is on its way while this one is multiplied.  A third stage (two
+// tiles in flight) measured the same to 1 % at every grid size tried (alternating runs on one device), so the smaller
+// footprint stays: two workgroups fit a compute unit's LDS.
+constexpr int QR_XST = 2;
 constexpr int QR_LW = 4;               // wavefronts that only issue the LDS-DMA, one per SIMD
 constexpr size_t QR_LDS = (size_t)QR_XST * QR_XSB + 2 * QR_BN * 4 * 8;
 
@@ -112,7 +115,8 @@ __global__ __launch_bounds__(64 * (MW + QR_LW)) void gemm_q4k_kernel(GemmQ4kArgs
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xk + xsrc[n]),
                                                  (__attribute__((address_space(3))) void *)(Xs + stage * QR_XSB + min(4 * n + lw, 32) * 1024), 16, 0, 0);
         };
-        constexpr int kOlder = 0x0F70 | (NI & 0xF) | (((NI >> 4) & 0x3) << 14); // all but the newest tile have landed
+        constexpr int kNewer = QR_XST == 3 ? NI : 0; // with three stages the newest tile may still be on its way
+        constexpr int kOlder = 0x0F70 | (kNewer & 0xF) | (((kNewer >> 4) & 0x3) << 14);
         auto publish = [&]() {
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_waitcnt(kOlder);
@@ -120,13 +124,13 @@ __global__ __launch_bounds__(64 * (MW + QR_LW)) void gemm_q4k_kernel(GemmQ4kArgs
             asm volatile("" ::: "memory");
         };
         issue_x(0, 0);
-        issue_x(1, min((int64_t)1, last));
+        if (QR_XST == 3) issue_x(1, min((int64_t)1, last));
         publish(); // super-block 0
-        int fill = 2;
+        int fill = QR_XST - 1;
         for (int64_t sb = 0; sb < last; sb++) {
             // stage `fill` held super-block sb - 1, read for the last time before the barrier just passed
-            issue_x(fill, min(sb + 2, last)); // past the end: the last one again, into a stage nobody reads
-            publish();                        // super-block sb + 1
+            issue_x(fill, min(sb + QR_XST - 1, last)); // past the end: the last one again, into a stage nobody reads
+            publish();                                 // super-block sb + 1
             fill = fill == QR_XST - 1 ? 0 : fill + 1;
         }
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): nothing lands after the wavefront has ended
@@ -329,6 +333,7 @@ __global__ __launch_bounds__(64 * (MW + QR_LW)) void gemm_q4k_kernel(GemmQ4kArgs
         // stores, 256 bytes per activation row.
         constexpr int OLD = BM + 8; // halfs per staged row: rows 272 bytes apart spread the lane groups over the banks
         half_t *Os = (half_t *)smem;
+        static_assert((size_t)QR_BN * OLD * 2 <= (size_t)QR_XST * QR_XSB, "the staged output tile fits the activation stages");
         rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
             for (int a = 0; a < TA; a++) {
@@ -396,12 +401,12 @@ hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const
     const int64_t tiles_j = (p.N + QR_BN - 1) / QR_BN;
     g.tiles_j = (int)tiles_j;
     g.vec_out = p.o_is == 1 && p.o_js % 8 == 0 && p.o_bs % 8 == 0 && ((uintptr_t)out & 15u) == 0;
-    auto go = [&](auto kernel, int bm, int threads) -> hipError_t {
+    auto go = [&](auto kernel, int bm) -> hipError_t {
         const int64_t tiles_i = (p.M + bm - 1) / bm;
         if (tiles_i * tiles_j > 0x7fffffff) return hipErrorNotSupported;
         g.remap = (tiles_i * tiles_j) % 8 == 0;
         if (const hipError_t e = ensure_lds_limit<decltype(kernel)::value>(); e != hipSuccess) return e;
-        hipLaunchKernelGGL(decltype(kernel)::value, dim3((unsigned)(tiles_i * tiles_j), (unsigned)p.stacks), dim3(threads), QR_LDS, stream, g);
+        hipLaunchKernelGGL(decltype(kernel)::value, dim3((unsigned)(tiles_i * tiles_j), (unsigned)p.stacks), dim3(64 * (4 + QR_LW)), QR_LDS, stream, g);
         return hipGetLastError();
     };
     // Four multiplying wavefronts of 32 weight rows x 64 activation rows each; when the grid of 16-row wavefronts
@@ -409,8 +414,8 @@ hipError_t launch_gemm_q4k(const Problem &p, const void *A, const void *B, const
     // (8192 x 3072 at 64 / 128 rows: 15.7 / 16.8 us against 22.6 / 23.6; 3072 x 8192 at 256 rows: 35 against 52 us).
     const int64_t wgs_small = ((p.M + 63) / 64) * tiles_j;
     const bool small = g_gemm_q4k_cfg == 14 || (g_gemm_q4k_cfg == 0 && wgs_small <= dev.num_cus);
-    if (small) return go(std::integral_constant<void (*)(GemmQ4kArgs), &gemm_q4k_kernel<1, 4>>{}, 64, 512);
-    return go(std::integral_constant<void (*)(GemmQ4kArgs), &gemm_q4k_kernel<2, 4>>{}, 128, 512);
+    if (small) return go(std::integral_constant<void (*)(GemmQ4kArgs), &gemm_q4k_kernel<1, 4>>{}, 64);
+    return go(std::integral_constant<void (*)(GemmQ4kArgs), &gemm_q4k_kernel<2, 4>>{}, 128);
 }
 
 } // namespace rt
