@@ -87,19 +87,32 @@ class Runner:
 
     REGIONS = 11   # timed regions of `steps` launches each; the median is reported
 
+    MAX_COVER = 256  # untimed graph replays the host may put in front of a region to stay ahead of the device
+
     def time_steps(self, launch_step, steps, warmup, n_variants, stats=None):
         """Times `steps` calls of launch_step(i) after `warmup` untimed ones, REGIONS times over, each region
         between its own pair of HIP events on the launch stream, and returns the median region's
         (ms_per_step, mode); `stats`, a dict, also receives the fastest and slowest region and the count.
-        The launches are captured into one HIP graph of whole rotations of the weight copies (20 launches
-        or more) when capture works, so the host's launch rate does not bound a ~6 us kernel; a region is
-        steps // 20 replays plus the remaining launches one by one, behind one untimed replay that keeps the
-        device busy while the host enqueues the region.  Otherwise all are issued one by one."""
+
+        The host needs longer to enqueue a launch than a ~6 us kernel runs, so a region must not contain the
+        host's enqueue time.  The launches are captured once into a HIP graph of whole rotations of the weight
+        copies (20 launches or more).  Two kinds of region:
+          "stream behind a hipgraph cover": untimed replays of that graph keep the device busy while the host
+              enqueues the first event, the `steps` launches one by one as any caller would, and the second
+              event; by the time the cover has drained, the host is far enough ahead that the device never waits
+              for it: a region counts only if the device still had a backlog when the last launch had been
+              enqueued, else all regions are taken again behind twice the cover.  Used when at most MAX_COVER
+              replays give that head start (any kernel of a few microseconds or more).
+          "hipgraph": otherwise (kernels much shorter than an enqueue) the region is steps // 20 replays of the
+              graph plus the remaining launches one by one, behind one untimed replay.  Launches inside a
+              replay follow each other about 0.2 us more slowly than launches in a stream, and a replay adds
+              about 5 us at its start and end.
+        Without graph capture all launches are issued one by one."""
         torch = self.torch
         for i in range(warmup):
             launch_step(i % n_variants)
         torch.cuda.synchronize()
-        mode, graph = "stream", None
+        mode, graph, covers = "stream", None, 0
         per_graph = n_variants * -(-20 // n_variants)  # at least 20 launches per replay
         try:
             graph = torch.cuda.CUDAGraph()
@@ -113,31 +126,67 @@ class Runner:
             sys.stderr.write(f"bench: graph capture unavailable ({type(e).__name__}: {e}); plain launches\n")
             graph = None
             torch.cuda.synchronize()
-        times = []
-        for _ in range(self.REGIONS):
+        if graph is not None:
+            # what the host needs per enqueue and the device per step: the cover must outlast the difference
+            t0 = time.perf_counter()
+            for i in range(per_graph):
+                launch_step(i % n_variants)
+            host_s = (time.perf_counter() - t0) / per_graph
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            graph.replay()
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            dev_s = e0.elapsed_time(e1) * 1e-3 / per_graph
+            covers = 1 + int(-(-max(0.0, steps * (1.5 * host_s - dev_s) + 100e-6) // (per_graph * dev_s)))
+
+        def region(covers):
+            """One timed region: (ms per step, seconds the device still had to run when the host had enqueued it all)."""
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
-            if graph is not None:
-                # one untimed replay ahead of the first event: the device is still busy with it while the host
-                # enqueues the event and the timed replays, so a short region (the driver's --steps 20 is a single
-                # replay) holds its `steps` launches back to back like a long one, not the host's enqueue latency too
-                graph.replay()
-            e0.record()
-            if graph is not None:
+            if covers:
+                for _ in range(covers):
+                    graph.replay()
+                e0.record()
+                for i in range(steps):
+                    launch_step(i % n_variants)
+            elif graph is not None:
+                graph.replay()  # the device is still busy with it while the host enqueues the event and the timed replays
+                e0.record()
                 full, rest = divmod(steps, per_graph)
                 for _ in range(full):
                     graph.replay()
                 for i in range(rest):
                     launch_step(i % n_variants)
             else:
+                e0.record()
                 for i in range(steps):
                     launch_step(i % n_variants)
             e1.record()
+            t_enq = time.perf_counter()
             torch.cuda.synchronize()
-            times.append(e0.elapsed_time(e1) / steps)
+            return e0.elapsed_time(e1) / steps, time.perf_counter() - t_enq
+
+        # A covered region counts only if the device was still well behind the host when the last launch had been
+        # enqueued (the backlog shrinks all the way through a region, so then it never ran dry).  If one was not,
+        # all regions are taken again behind twice the cover; past MAX_COVER the graph replays are timed instead.
+        times = []
+        while graph is not None and covers:
+            if covers > self.MAX_COVER:
+                covers = 0
+                break
+            runs = [region(covers) for _ in range(self.REGIONS)]
+            if all(backlog >= max(200e-6, 10 * dev_s) for _, backlog in runs):
+                times, mode = [ms for ms, _ in runs], "stream behind a hipgraph cover"
+                break
+            covers *= 2
+        if not times:
+            times = [region(0)[0] for _ in range(self.REGIONS)]
         times.sort()
         if stats is not None:
-            stats.update(regions=len(times), ms_per_step_min=times[0], ms_per_step_max=times[-1])
+            stats.update(regions=len(times), ms_per_step_min=times[0], ms_per_step_max=times[-1], cover_replays=covers)
         return times[len(times) // 2], mode
 
 
@@ -695,8 +744,8 @@ def cpu_baseline(O, wbuf, x, bias, budget_s=1.5):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-secondary", action="store_true", help="only the headline workload")
     ap.add_argument("--gemm-only", action="store_true",
                     help="run only the two C4 GEMM workloads (f16 and Q8_0H weights) and print their lines; for profiling")
@@ -808,6 +857,7 @@ def main():
             "weight_copies_rotated": head["copies"],
             "launch": head["mode"],
             "timed_regions": head["stats"]["regions"],
+            "untimed_graph_replays_ahead_of_a_region": head["stats"]["cover_replays"],
             "ms_per_step_is": "median over the timed regions of `steps` launches each",
             "ms_per_step_min": head["stats"]["ms_per_step_min"],
             "ms_per_step_max": head["stats"]["ms_per_step_max"],
