@@ -823,17 +823,18 @@ def main():
         warm = bench_q8_gemv(r, O, 1, sec_steps, max(20, args.warmup // 4), copies=1)
         warm.pop("inputs"), warm.pop("stats")
         secondary.append({"workload": "C2 Q8_0 GEMV M=1, warm: one weight copy, resident in the Infinity Cache (not HBM)",
-                          "value": round(warm["gbps"], 1), "unit": "GB/s", "ms_per_step": warm["ms"]})
+                          "value": round(warm["gbps"], 1), "unit": "GB/s", "ms_per_step": warm["ms"], "timing": warm["mode"]})
         for M in (4, 8):
             s = bench_q8_gemv(r, O, M, sec_steps, max(20, args.warmup // 4), seed=M)
             s.pop("inputs"), s.pop("stats")
             secondary.append({"workload": f"C2 Q8_0 GEMV M={M}", "value": round(s["gbps"], 1), "unit": "GB/s",
-                              "ms_per_step": s["ms"], "frac_hbm_peak": round(s["gbps"] / HBM_PEAK_GBPS, 4)})
+                              "ms_per_step": s["ms"], "timing": s["mode"], "frac_hbm_peak": round(s["gbps"] / HBM_PEAK_GBPS, 4)})
         gsteps = max(50, args.steps // 40)
         for g in (gemm_f16, bench_q8_gemm(r, O, gsteps, 10),
                   bench_q8_gemm(r, O, gsteps, 10, act=r.ffi.RT_ACT_GELU)):
             secondary.append({"workload": g["workload"], "value": round(g["tflops"], 1), "unit": "TFLOP/s",
-                              "ms_per_step": g["ms"], "frac_mfma_f16_peak": round(g["tflops"] / MFMA_F16_PEAK_TFLOPS, 4)})
+                              "ms_per_step": g["ms"], "timing": g["mode"],
+                              "frac_mfma_f16_peak": round(g["tflops"] / MFMA_F16_PEAK_TFLOPS, 4)})
 
         secondary += bench_elementwise(r, O)
         secondary += other_configs(r, O)
