@@ -590,7 +590,18 @@ def other_configs(r: Runner, O):
     out += bench_attention(r, O)
     out.append(bench_decoder_layer(r, O))
     out.append(bench_decoder_layer(r, O, fused_qkv=True))
-    out += bench_q4k(r, O, (1, 16, 256), 200)
+    out += bench_q4k(r, O, (1, 16, 128, 256), 200)
+    # a short prompt against the C4 up-projection: 128 activation rows run on 64-row weight tiles so that every
+    # compute unit has a workgroup (160 workgroups; the 160-row tile would leave 64)
+    rng = np.random.default_rng(8)
+    w = (rng.standard_normal((10240, 2560)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((1, 128, 2560)).astype(np.float16)
+    bias = rng.standard_normal(10240).astype(np.float16)
+    for name, lhs, dt, wbytes in (("f16", w.astype(np.float16), ffi.RT_F16, 10240 * 2560 * 2),
+                                  ("Q8_0H", O.make_q8_0h(w), ffi.RT_Q8_0H, 10240 * 2560 * 17 // 16)):
+        out.append(bench_generic(r, O, f"C4 up at 128 rows: X[128x2560] f16 . {name} W[10240x2560]^T + bias", lhs, dt,
+                                 (10240, 2560), x, x.shape, bias, (False, True, True), np.float16, 2.0 * 128 * 10240 * 2560,
+                                 wbytes + (128 * 2560 + 10240 + 128 * 10240) * 2, 100, 2e-2))
     return out
 
 
@@ -615,7 +626,7 @@ def c3_products(r: Runner, O):
 
 
 def bench_q4k(r: Runner, O, rows, steps):
-    """BASELINE configs[4]: Q4_K W[8192x3072] against 1 / 16 (streaming kernel) and 256 (tiled kernel) f16 rows."""
+    """BASELINE configs[4]: Q4_K W[8192x3072] against 1 / 16 (streaming kernel) and 128 / 256 (tiled kernel) f16 rows."""
     ffi, out = r.ffi, []
     rng = np.random.default_rng(5)
     blocks = O.q4k_quantize((rng.standard_normal((8192, 3072)) * 0.02).astype(np.float32))
