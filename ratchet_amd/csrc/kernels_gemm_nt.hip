@@ -1048,6 +1048,12 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
         // the narrow tiles take as deep a ring as the LDS holds: a stage has only 8 or 12 KB of weights, and what a compute
         // unit has in flight is what it can pull (10240 x 2560 f16 weights, 40 / 64 activation rows, three stages -> six:
         // 22.7 / 23.6 -> 20.0 / 22.1 us with the weights in HBM, 16.3 / 16.8 -> 14.8 / 15.7 from the Infinity Cache)
+        if (dl_f16 && bm == 64 && p.N <= 64) {
+            // up to 64 activation rows: half the activation tile, a stage of 16 KB and nine of them (40 / 64 rows:
+            // 20.0 / 22.1 -> 18.3 / 20.5 us with the weights in HBM, 14.8 / 15.7 -> 12.6 / 13.6 from the Infinity Cache)
+            g.tiles_j = 1;
+            return launch_nt_dl<64, 64, 9, 2>(g, p.stacks, stream);
+        }
         if (dl_f16) return bm == 64 ? launch_nt_dl<64, BN, 6, 2>(g, p.stacks, stream) : launch_nt_dl<96, BN, 5, 2>(g, p.stacks, stream);
         return bm == 64 ? launch_nt_q8w<64, BN, 4>(g, p.stacks, stream) : launch_nt_q8w<96, BN, 4>(g, p.stacks, stream);
     }
