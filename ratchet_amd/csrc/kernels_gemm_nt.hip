@@ -1055,6 +1055,11 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
             return launch_nt_dl<64, 64, 9, 2>(g, p.stacks, stream);
         }
         if (dl_f16) return bm == 64 ? launch_nt_dl<64, BN, 6, 2>(g, p.stacks, stream) : launch_nt_dl<96, BN, 5, 2>(g, p.stacks, stream);
+        if (bm == 64 && p.N <= 64) {
+            // up to 64 activation rows: half the activation tile is half the MFMAs and folds of a workgroup
+            g.tiles_j = 1;
+            return launch_nt_q8w<64, 64, 4>(g, p.stacks, stream);
+        }
         return bm == 64 ? launch_nt_q8w<64, BN, 4>(g, p.stacks, stream) : launch_nt_q8w<96, BN, 4>(g, p.stacks, stream);
     }
     if (dl_f16) {

@@ -283,14 +283,18 @@ RT_TUNABLE(g_gemv_disable_mfma, 0);
 // such requirement.
 // A few more activation vectors than one streaming launch takes: one launch per 16 of them.  Each
 // launch streams the weights again (after the first mostly from the Infinity Cache), which still beats
-// the tiled kernels while the MFMA work is small: measured at 10240 x 2560 Q8_0H, 17 / 32 vectors take
-// 18 / 20 us (48 / 64: 29 / 38) against 21 us tiled at any count up to 64, and at 8192 x 3072 Q4_K
-// 17 / 32 vectors take 12 / 14 us (48: 21) against 15 us tiled: the tiled kernels take over from 33.
+// the tiled kernels while the MFMA work is small: measured at 8192 x 3072 Q4_K, 17 / 32 vectors take
+// 12 / 14 us (48: 21) against 15 us tiled: the tiled kernels take over from 33.  (10240 x 2560 Q8_0H:
+// 18 / 20 us, 48 / 64 vectors 29 / 38.)
 hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                hipStream_t stream, const DeviceInfo &dev) {
     const bool q8 = p.a_dt == RT_Q8_0H, q4 = p.a_dt == RT_Q4_K;
     if ((!q8 && !q4) || p.act_dt != RT_F16 || g_gemv_disable_mfma) return hipErrorNotSupported;
     if (p.N <= 16 || p.N > 32) return hipErrorNotSupported;
+    // Q8_0H weights with enough rows that their 64 x 64 tiles give half of the compute units a workgroup are faster on
+    // the tiled kernel (10240 x 2560: 15.7 / 16.2 us at 17 / 32 vectors); with fewer rows (2560 x 2560: 40 tiles) the
+    // streaming launches stay ahead
+    if (q8 && p.K % 256 == 0 && p.stacks == 1 && (p.M + 63) / 64 >= dev.num_cus / 2) return hipErrorNotSupported;
     for (int64_t j0 = 0; j0 < p.N; j0 += 16) {
         Problem c = p;
         c.N = p.N - j0 < 16 ? p.N - j0 : 16;

@@ -702,7 +702,9 @@ def test_f16_nt_gemm_stack_broadcast(device, oracle):
 
 def test_q8_nt_gemm_edges(device, oracle):
     for i, (S, M, N, K) in enumerate([(1, 160, 64, 64), (1, 161, 65, 96), (1, 333, 200, 160), (2, 170, 70, 32),
-                                      (1, 1000, 129, 2560), (1, 2560, 77, 1024), (2, 200, 100, 256), (3, 161, 64, 512)]):
+                                      (1, 1000, 129, 2560), (1, 2560, 77, 1024), (2, 200, 100, 256), (3, 161, 64, 512),
+                                      # 17..64 activation rows against many weight rows: 64 x 64 tiles instead of streaming launches
+                                      (1, 8300, 33, 512), (1, 8200, 24, 256), (1, 10240, 17, 2560)]):
         rng = np.random.default_rng(700 + i)
         w = (rng.standard_normal((S, M, K)) * 0.02).astype(np.float32)
         buf = oracle.make_q8_0h(w)
@@ -723,7 +725,7 @@ def test_q8_tiled_one_hot_is_bit_exact_dequant(device, oracle):
     """The tiled Q8_0H kernels (K % 256 == 0 and not) with one-hot activations: each output is one
     dequantized weight, which must match the oracle's dequantizer bit for bit, -128 included."""
     rng = np.random.default_rng(720)
-    for N, K, M in [(320, 256, 64), (200, 512, 100), (170, 96, 70), (2100, 256, 1300), (9000, 256, 200)]:  # the last two: 160- and 96-row tiles
+    for N, K, M in [(320, 256, 64), (200, 512, 100), (170, 96, 70), (2100, 256, 1300), (9000, 256, 200), (9000, 256, 20)]:  # 160-row, 96-row and 64 x 64 tiles last
         buf = q8_weight(oracle, rng, N, K, DType.Q8_0H)
         buf[: N * K][3::89] = 0x80
         dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
