@@ -966,7 +966,7 @@ static bool nt_orient(Problem &p) {
 uint64_t gemm_nt_workspace_bytes(const Problem &p0, const DeviceInfo &dev) {
     Problem p = p0;
     nt_orient(p);
-    if (p.a_ks != 1 || p.b_ks != 1 || p.M < 160 || p.N < 8) return 0;
+    if (p.a_ks != 1 || p.b_ks != 1 || p.M < 160 || p.N < 5) return 0;
     const int ks = gemm_nt_ksplit(p, dev);
     return ks > 1 ? (uint64_t)p.stacks * ks * p.M * p.N * sizeof(float) : 0;
 }
@@ -987,7 +987,7 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
     if (q8 ? (p.K % 32 != 0) : ((p.a_rs * 2) % 16 != 0 || (p.a_bs * 2) % 16 != 0)) return hipErrorNotSupported;
     // small problems do not fill the tiles; the generic kernel handles them (at 10240 x 2560 f16 weights it takes
     // 19.7 us for 8 activation rows and 33 us for 16..48, the 64-row tiles here 17.4 us for any count up to 64)
-    if (p.M < 160 || p.N < 8) return hipErrorNotSupported;
+    if (p.M < 160 || p.N < 5) return hipErrorNotSupported;
 
     GemmNtArgs g{};
     g.A = A, g.B = (const half_t *)B, g.bias = (const half_t *)bias, g.out = (half_t *)out;
