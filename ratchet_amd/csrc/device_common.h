@@ -148,6 +148,8 @@ hipError_t launch_gemv(const Problem &p, const void *A, const void *B, const voi
                        hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_q8h_mfma(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                 hipStream_t stream, const DeviceInfo &dev);
+hipError_t launch_gemv_q8h_quad(const Problem &p, const void *A, const void *B, const void *bias, void *out,
+                                hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_q8h_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                                   hipStream_t stream, const DeviceInfo &dev);
 hipError_t launch_gemv_float_rowdot(const Problem &p, const void *A, const void *B, const void *bias, void *out,

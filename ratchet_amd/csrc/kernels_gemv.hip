@@ -313,9 +313,11 @@ hipError_t launch_gemv_chunked(const Problem &p, const void *A, const void *B, c
 hipError_t launch_gemv(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                        hipStream_t stream, const DeviceInfo &dev) {
     if (p.kernel == RT_KERNEL_GEMV_Q8 && p.a_dt == RT_Q8_0H && !g_gemv_disable_mfma) {
-        // f16 activations, one or two vectors: the row-streaming kernel; then the matrix-core kernel;
-        // shapes both decline fall through
+        // f16 activations, one or two vectors: the row-streaming kernel; three or four: the row-streaming kernel on
+        // the 4x4x4 matrix instruction; then the matrix-core kernel; shapes all of them decline fall through
         hipError_t e = launch_gemv_q8h_rowdot(p, A, B, bias, out, stream, dev);
+        if (e != hipErrorNotSupported) return e;
+        e = launch_gemv_q8h_quad(p, A, B, bias, out, stream, dev);
         if (e != hipErrorNotSupported) return e;
         e = launch_gemv_q8h_mfma(p, A, B, bias, out, stream, dev);
         if (e != hipErrorNotSupported) return e;

@@ -274,6 +274,51 @@ def test_q8_row_streaming_one_and_two_vectors(device, oracle):
             assert np.array_equal(got, dq[:, cols].T.astype(np.float16)), (N, K, M)
 
 
+def test_q8_row_streaming_three_and_four_vectors(device, oracle):
+    """Q8_0H weights against three or four vectors, K a multiple of 256 up to 4096 and at least 16 rows per compute
+    unit take the row-streaming kernel on the 4x4x4 matrix instruction: every step count (K = 256 .. 4096), row
+    counts off the 16 rows of a workgroup and off the four of a wavefront, stacks of weights and of activations with
+    broadcast either way, the bias along the rows (trans_out) and along the vectors, a fused activation; then
+    one-hot activations, bit for bit, with -128 planted."""
+    dt = DType.Q8_0H
+    cases = [(1, 3 + (k & 1), 4096 + 3 * k, 256 * k) for k in range(1, 17)]
+    cases += [(1, 4, 10240, 2560), (1, 3, 4097, 2560), (2, 4, 2069, 768), (3, 3, 1400, 1280)]
+    for i, (S, M, N, K) in enumerate(cases):
+        rng = np.random.default_rng(2600 + i)
+        for ws, xs_ in ((S, S), (1, S), (S, 1)) if S > 1 else ((1, 1),):
+            w = (rng.standard_normal((ws, N, K)) * 0.05).astype(np.float32)
+            buf = oracle.make_q8_0h(w)
+            x = rng.standard_normal((xs_, M, K)).astype(np.float16)
+            for to in (True, False):
+                bias = rng.standard_normal(N if to else M).astype(np.float16) if (i + to) % 3 else None
+                got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (ws, N, K)), Tensor.from_data(x),
+                                 None if bias is None else Tensor.from_data(bias), False, True, to)
+                want = oracle.matmul_ref(buf, oracle.Q8_0H, (ws, N, K), x, oracle.F16, x.shape, bias, False, True, to)
+                check(oracle, got, want, DType.F16, (S, ws, xs_, M, N, K, to))
+    # GELU / SiLU behind the Linear, fused
+    rng = np.random.default_rng(2680)
+    N, K = 4200, 1024
+    buf = oracle.make_q8_0h((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    x = rng.standard_normal((1, 4, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    for name, act in (("gelu", oracle.ACT_GELU), ("silu", oracle.ACT_SILU)):
+        y = getattr(Tensor.from_quantized(buf, dt, (N, K)).to(device).gemm(
+            Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device), False, True, True), name)().resolve()
+        want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, bias, False, True, True, act=act)
+        assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
+    # one-hot: the dequantized weight, bit for bit
+    for N, K in ((4099, 2560), (4200, 256), (4096, 4096)):
+        buf = q8_weight(oracle, rng, N, K, dt)
+        buf[: N * K][5::97] = 0x80
+        dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
+        for M in (3, 4):
+            cols = np.concatenate([[5 + 97 * 2], rng.integers(0, K, size=M)])[:M]
+            x = np.zeros((M, K), dtype=np.float16)
+            x[np.arange(M), cols] = 1
+            got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (N, K)), Tensor.from_data(x), None, False, True, True)
+            assert np.array_equal(got, dq[:, cols].T.astype(np.float16)), (N, K, M)
+
+
 @pytest.mark.parametrize("dt", [DType.Q8_0H, DType.Q8_0F], ids=["q8_0h", "q8_0f"])
 def test_q8_one_hot_is_bit_exact_dequant(device, oracle, dt):
     """A one-hot activation selects one dequantized weight per row: the GEMV / GEMM
