@@ -87,6 +87,27 @@ class Runner:
 
     REGIONS = 11   # timed regions of `steps` launches each; the median is reported
 
+    def wall_clock_ms_per_step(self, launch_step, n_variants, replays=2000):
+        """A cross-check of the event timing that uses no HIP event: `replays` replays of a HIP graph of one
+        rotation of the weight copies (20 launches or more) between two device synchronisations, timed with the
+        host's clock.  The host enqueues a replay much faster than the device runs it, so the device is never idle
+        in between; the figure includes the ends of the replays (about 0.2 us per launch more than launches that
+        follow each other in a stream)."""
+        torch = self.torch
+        per_graph = n_variants * -(-20 // n_variants)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(per_graph):
+                launch_step(i % n_variants)
+        for _ in range(10):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / (replays * per_graph), replays * per_graph
+
     MAX_COVER = 256  # untimed graph replays the host may put in front of a region to stay ahead of the device
 
     def time_steps(self, launch_step, steps, warmup, n_variants, stats=None):
@@ -190,7 +211,7 @@ class Runner:
         return times[len(times) // 2], mode
 
 
-def bench_q8_gemv(r: Runner, O, M, steps, warmup, seed=0, copies=None):
+def bench_q8_gemv(r: Runner, O, M, steps, warmup, seed=0, copies=None, wall_clock=False):
     """C2.  `copies` = 1 measures the warm case (the one weight stays in the 256 MB Infinity Cache); the
     default rotates enough copies that every launch streams its weight from HBM."""
     N, K = 10240, 2560
@@ -208,6 +229,9 @@ def bench_q8_gemv(r: Runner, O, M, steps, warmup, seed=0, copies=None):
     desc = r.ffi.make_desc(r.ffi.RT_Q8_0H, (N, K), r.ffi.RT_F16, (1, M, K), False, True, True, r.ffi.RT_F16, (N,))
     stats = {}
     ms, mode = r.time_steps(lambda i: r.enqueue(desc, ws[i], xd, bd, outs[i]), steps, warmup, copies, stats)
+    if wall_clock:
+        stats["wall_clock_ms_per_step"], stats["wall_clock_launches"] = r.wall_clock_ms_per_step(
+            lambda i: r.enqueue(desc, ws[i], xd, bd, outs[i]), copies)
     # parity of what was just timed, against the oracle on the same inputs
     got = outs[(steps - 1) % copies].cpu().numpy().view(np.float16).reshape(1, M, N)
     ref = O.matmul_ref(wbuf, O.Q8_0H, (N, K), x, O.F16, x.shape, bias, False, True, True)
@@ -673,12 +697,23 @@ def read_calibration(r: Runner, O, steps, warmup):
     out = r.torch.empty(N * 2, dtype=r.torch.uint8, device="cuda:0")
     store_out = r.torch.empty(4 * 4 * (-(-nbytes // 5120 // 4) + 1), dtype=r.torch.uint8, device="cuda:0")  # whole workgroups of 4
     desc = r.ffi.make_desc(r.ffi.RT_Q8_0H, (N, K), r.ffi.RT_F16, (1, 1, K), False, True, True, r.ffi.RT_F16, (N,))
+    lib_src = [w[:nbytes].view(r.torch.float32) for w in ws]
+    lib_dst = r.torch.empty_like(lib_src[0])
+    lib_sum = lambda i: r.torch.sum(lib_src[i])
+    lib_mat = [w[:10240 * 1360 * 2].view(r.torch.float16).view(10240, 1360) for w in ws]
+    lib_vec = r.torch.ones(1360, dtype=r.torch.float16, device="cuda:0")
+    lib_mv = lambda i: r.torch.mv(lib_mat[i], lib_vec)
     rows = []
     for name, step, nb in (
             ("empty kernel (one wavefront)", lambda i: ok(P.probe_empty(vp(sink.data_ptr()), stream())), 0),
             ("read only, consecutive addresses", lambda i: ok(P.probe_read_linear(vp(ws[i].data_ptr()), nbytes, 0, vp(sink.data_ptr()), stream())), nbytes),
             ("read only, consecutive addresses, non-temporal loads", lambda i: ok(P.probe_read_linear(vp(ws[i].data_ptr()), nbytes, 1, vp(sink.data_ptr()), stream())), nbytes),
             ("read (non-temporal) + 4 bytes stored per wavefront of 5 KiB", lambda i: ok(P.probe_read_linear_store(vp(ws[i].data_ptr()), nbytes, vp(store_out.data_ptr()), stream())), nbytes),
+            # passes over the same bytes by kernels this repository did not write: torch's reduction, the vendor BLAS's
+            # GEMV reading the buffer as an f16 [10240 x 1360] matrix, the runtime's device copy (reads and writes)
+            ("library: torch.sum over the weight as f32 (read only)", lambda i: lib_sum(i), nbytes),
+            ("library: torch.mv, the weight as f16 [10240 x 1360] (vendor BLAS GEMV, read only)", lambda i: lib_mv(i), 10240 * 1360 * 2),
+            ("library: device-to-device copy of the weight (reads and writes the bytes)", lambda i: lib_dst.copy_(lib_src[i], non_blocking=True), 2 * nbytes),
             ("read only, 16 rows x 64 bytes per load (the int8 codes alone)", lambda i: ok(P.probe_read_rows16(vp(ws[i].data_ptr()), N, K, vp(sink.data_ptr()), stream())), N * K),
             ("Q8_0H GEMV M=1 (the headline)", lambda i: r.enqueue(desc, ws[i], xd, bd, out), gemv_bytes(1, N, K))):
         stats = {}
@@ -729,6 +764,48 @@ def issue_calibration(r: Runner):
     return {"issue_calibration": rows, "trips": iters, "wavefronts_per_simd": 1}
 
 
+def gemm_ablation(r: Runner):
+    """What bounds the f16 tiled GEMM at X[512 x 2560] . W[10240 x 2560]^T + bias: the shipped kernel next to timing-only
+    builds of the same source with parts left out (their results are wrong; ratchet_amd/libratchet_probes.so holds them,
+    built from csrc/kernels_gemm_nt.hip with RT_NT_ABLATION set).  Same timing as every other workload here."""
+    torch = r.torch
+    M, N, K = 512, 10240, 2560
+    rng = np.random.default_rng(5)
+    wd = r.upload((rng.standard_normal((N, K)) * 0.02).astype(np.float16))
+    xd = r.upload(rng.standard_normal((1, M, K)).astype(np.float16))
+    bd = r.upload(rng.standard_normal(N).astype(np.float16))
+    out = torch.empty(M * N * 2, dtype=torch.uint8, device="cuda:0")
+    desc = r.ffi.make_desc(r.ffi.RT_F16, (N, K), r.ffi.RT_F16, (1, M, K), False, True, True, r.ffi.RT_F16, (N,))
+    P = ctypes.CDLL(os.path.join(ROOT, "ratchet_amd", "libratchet_probes.so"))
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+
+    def variant(mask):
+        fn = getattr(P, f"probe_gemm_nt_ablation_{mask}")
+        fn.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+
+        def step(i):
+            rc = fn(vp(wd.data_ptr()), vp(xd.data_ptr()), vp(bd.data_ptr()), vp(out.data_ptr()), N, M, K,
+                    vp(torch.cuda.current_stream().cuda_stream))
+            if rc != 0:
+                raise RuntimeError(f"probe launch failed: hipError {rc}")
+        return step
+
+    rows = []
+    for name, step in (("the kernel as shipped", lambda i: r.enqueue(desc, wd, xd, bd, out)),
+                       ("no output stores", variant(8)),
+                       ("no fragment reads (tile loads + MFMAs + barriers + output)", variant(4)),
+                       ("no tile loads, no output (fragment reads + MFMAs + barriers)", variant(9)),
+                       ("MFMAs + barriers only (no tile loads, no fragment reads, no output)", variant(13)),
+                       ("tile loads + barriers only (no MFMAs, no fragment reads, no output)", variant(14)),
+                       ("barriers + output only (no tile loads, no MFMAs, no fragment reads)", variant(7)),
+                       ("barriers only", variant(15))):
+        stats = {}
+        ms, mode = r.time_steps(step, 100, 10, 1, stats)
+        rows.append({"variant": name, "us_per_launch": round(ms * 1e3, 2), "us_min": round(stats["ms_per_step_min"] * 1e3, 2),
+                     "timing": mode})
+    return {"gemm_ablation": rows, "shape": "X[512x2560] f16 . W[10240x2560]^T f16 + bias", "kernel": "gemm_nt_dl_kernel<160, 128, 3, 2>"}
+
+
 def cpu_baseline(O, wbuf, x, bias, budget_s=1.5):
     """The oracle's reference path on the host cores, same inputs: median of >= 3 runs.  Returns
     (seconds, runs) for the whole path (dequantize W to f32, f32 GEMV, bias, cast) and the same for the
@@ -770,6 +847,8 @@ def main():
                     help="only time an empty launch and read-only passes over the rotated weight copies next to the GEMV")
     ap.add_argument("--issue-calibration", action="store_true",
                     help="time a wavefront's MFMAs, packed vector instructions and LDS fragment reads alone and mixed, and print the table")
+    ap.add_argument("--gemm-ablation", action="store_true",
+                    help="time the f16 tiled GEMM at the configs[3] shape next to timing-only builds of it with parts left out")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 20 device-to-device copies of 256 MiB (reference dispatches for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -797,6 +876,10 @@ def main():
         print(json.dumps(issue_calibration(r)))
         return 0
 
+    if args.gemm_ablation:
+        print(json.dumps(gemm_ablation(r)))
+        return 0
+
     if args.read_calibration:
         print(json.dumps(read_calibration(r, O, min(args.steps, 2000), min(args.warmup, 100))))
         return 0
@@ -821,7 +904,7 @@ def main():
         print(json.dumps(bench_q4k(r, O, (256,), 100)[0]))
         return 0
 
-    head = bench_q8_gemv(r, O, 1, args.steps, args.warmup)
+    head = bench_q8_gemv(r, O, 1, args.steps, args.warmup, wall_clock=True)
     wbuf, x, bias = head.pop("inputs")
     (cpu_s, cpu_n), (cpu_am_s, cpu_am_n) = cpu_baseline(O, wbuf, x, bias)
 
@@ -874,6 +957,9 @@ def main():
             "ms_per_step_min": head["stats"]["ms_per_step_min"],
             "ms_per_step_max": head["stats"]["ms_per_step_max"],
             "max_rel_err_vs_oracle": head["err"],
+            # no HIP event involved: host clock around 2000 replays of a graph of one rotation, between two synchronisations
+            "wall_clock_ms_per_step": head["stats"]["wall_clock_ms_per_step"],
+            "wall_clock_launches": head["stats"]["wall_clock_launches"],
         },
         "roofline": {
             "bound": "hbm",

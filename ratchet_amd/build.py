@@ -21,6 +21,8 @@ LIB = os.path.join(HERE, "libratchet_hip.so")
 PROBES_SRC = "bench_probes.hip"
 PROBES_LIB = os.path.join(HERE, "libratchet_probes.so")
 ARCH = "gfx950"
+# timing-only builds of the f16 tiled GEMM (bit mask: 1 no tile loads, 2 no MFMAs, 4 no fragment reads, 8 no output)
+NT_ABLATIONS = (4, 7, 8, 9, 13, 14, 15)
 
 SOURCES = ["api.cpp", "spec.cpp", "gguf.cpp", "kernels_blocks.hip", "kernels_softmax.hip", "kernels_unary.hip", "kernels_attention.hip", "kernels_gemv.hip", "kernels_gemv_mfma.hip", "kernels_gemv_rowdot.hip", "kernels_gemv_quad.hip", "kernels_gemv_rowfloat.hip",
     "kernels_gemv_q4k_mfma.hip", "kernels_gemv_q4k_rowdot.hip", "kernels_gemm.hip", "kernels_gemm_f32.hip", "kernels_gemm_q4k.hip",
@@ -69,6 +71,34 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
+def build_probes(force: bool = False) -> str:
+    """libratchet_probes.so: bench_probes.hip plus one timing-only build of kernels_gemm_nt.hip per entry of
+    NT_ABLATIONS (its namespace renamed, so the builds do not collide), for bench.py's calibration flags."""
+    os.makedirs(OBJ, exist_ok=True)
+    probes_src, nt_src = os.path.join(CSRC, PROBES_SRC), os.path.join(CSRC, "kernels_gemm_nt.hip")
+    deps = [probes_src, nt_src, os.path.abspath(__file__)] + [os.path.join(CSRC, h) for h in HEADERS]
+    if not (force or _stale(PROBES_LIB, deps)):
+        return PROBES_LIB
+
+    def one(job):
+        src, obj, extra = job
+        res = subprocess.run([hipcc(), *FLAGS, *extra, "-c", src, "-o", obj], capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {os.path.basename(src)} {' '.join(extra)}:\n{res.stderr}")
+        return obj
+
+    jobs = [(probes_src, os.path.join(OBJ, "bench_probes.o"), [])]
+    for mask in NT_ABLATIONS:
+        jobs.append((nt_src, os.path.join(OBJ, f"nt_ablation_{mask}.o"),
+                     [f"-DRT_NT_ABLATION={mask}", f"-Drt=rt_nt_ablation_{mask}", f"-DRT_NT_ABL_ENTRY=probe_gemm_nt_ablation_{mask}"]))
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
+        objs = list(ex.map(one, jobs))
+    res = subprocess.run([hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", PROBES_LIB, *objs], capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link of the probes failed:\n{res.stderr}")
+    return PROBES_LIB
+
+
 def build(force: bool = False, verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
@@ -78,12 +108,10 @@ def build(force: bool = False, verbose: bool = True) -> str:
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"link failed:\n{res.stderr}")
-    probes_src = os.path.join(CSRC, PROBES_SRC)
-    if force or _stale(PROBES_LIB, [probes_src, os.path.abspath(__file__)]):
-        cmd = [hipcc(), *FLAGS, "-shared", probes_src, "-o", PROBES_LIB]
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        if res.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {PROBES_SRC}:\n{res.stderr}")
+    try:
+        build_probes(force)
+    except RuntimeError as e:  # measurement probes only: the product does not depend on them
+        sys.stderr.write(f"warning: {e}\n")
     if verbose:
         print(f"built {LIB}")
     return LIB

@@ -10,6 +10,10 @@
 
 typedef uint32_t probe_u4 __attribute__((ext_vector_type(4)));
 
+// The timing-only builds of kernels_gemm_nt.hip that this library also holds (probe_gemm_nt_ablation_<mask>, see
+// build.py) refer to this function of the product library; the library's own copy keeps it self-contained.
+extern "C" uint64_t rt_q8_0_scale_offset(uint64_t numel) { return (numel + 255u) & ~(uint64_t)255u; }
+
 __global__ void probe_empty_kernel(uint32_t *sink) {
     if (sink == nullptr) sink[0] = 1; // never
 }

@@ -77,6 +77,12 @@ __device__ __forceinline__ void nt_tile_of(int64_t wg, int tiles_i, int tiles_j,
     ti = wg / tiles_j, tj = wg - ti * tiles_j;
 }
 
+// Timing-only variants of gemm_nt_dl_kernel for the measurement probes (a bit mask: 1 no tile loads, 2 no MFMAs,
+// 4 no fragment reads, 8 no output); the product is built with 0.
+#ifndef RT_NT_ABLATION
+#define RT_NT_ABLATION 0
+#endif
+
 constexpr int NT_BK = 64;
 constexpr int NT_LDK = NT_BK;     // halfs per LDS row: 128 B = 8 vectors of 16 B, no padding
 constexpr int NT_THREADS = 256;
@@ -429,6 +435,7 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
         }
         auto issue_tile = [&](int stage, int64_t k0) {
             half_t *st = ring + stage * STAGE_HALFS;
+            if (RT_NT_ABLATION & 1) return; // timing only: no tile loads
 #pragma unroll
             for (int c = 0; c < LCH; c++)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gp[c] + k0),
@@ -467,6 +474,7 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
         half8_t fa[TM], fb[TN];
     };
     auto read_one = [&](int stage, int kk, Frags &f, int i) {
+        if (RT_NT_ABLATION & 4) return; // timing only: no fragment reads
         const half_t *as = ring + stage * STAGE_HALFS + (wi * WM + fr) * NT_LDK + (((kk * 4 + fg) ^ swz) << 3);
         const half_t *bs = ring + stage * STAGE_HALFS + BM * NT_LDK + (wj * WN + fr) * NT_LDK + (((kk * 4 + fg) ^ swz) << 3);
         if (i < TM)
@@ -487,7 +495,12 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
         asm volatile("" ::: "memory");
     };
     meet(); // tile 0 visible
+#if RT_NT_ABLATION & 4
+    Frags f0 = {}, f1 = {};
+    asm volatile("" : "+v"(f0.fa[0]), "+v"(f1.fa[0]));
+#else
     Frags f0, f1;
+#endif
 #pragma unroll
     for (int i = 0; i < TM + TN; i++) read_one(0, 0, f0, i);
     int cur = 0, nxt = 1;
@@ -497,7 +510,7 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
     for (int64_t kt = 0; kt < nk; kt++) {
 #pragma unroll
         for (int m = 0; m < TM * TN; m++) {
-            acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f0.fb[m % TN], f0.fa[m / TN], acc[m / TN][m % TN], 0, 0, 0);
+            if (!(RT_NT_ABLATION & 2)) acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f0.fb[m % TN], f0.fa[m / TN], acc[m / TN][m % TN], 0, 0, 0);
             if (m % RS == RS - 1) {
                 if (m / RS < TM + TN) read_one(cur, 1, f1, m / RS);
                 __builtin_amdgcn_sched_barrier(0);
@@ -506,7 +519,7 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
         meet(); // tile kt + 1 visible
 #pragma unroll
         for (int m = 0; m < TM * TN; m++) {
-            acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f1.fb[m % TN], f1.fa[m / TN], acc[m / TN][m % TN], 0, 0, 0);
+            if (!(RT_NT_ABLATION & 2)) acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f1.fb[m % TN], f1.fa[m / TN], acc[m / TN][m % TN], 0, 0, 0);
             if (m % RS == RS - 1) {
                 if (m / RS < TM + TN) read_one(nxt, 0, f0, m / RS);
                 __builtin_amdgcn_sched_barrier(0);
@@ -517,6 +530,16 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __syncthreads();
+    if (RT_NT_ABLATION & 8) { // timing only: no output (one store per lane keeps the accumulators alive)
+        float v = 0.f;
+#pragma unroll
+        for (int a = 0; a < TM; a++)
+#pragma unroll
+            for (int b = 0; b < TN; b++) v += acc[a][b][0] + acc[a][b][1] + acc[a][b][2] + acc[a][b][3];
+        if (RT_NT_ABLATION & 4) v += (float)f0.fa[0][0] + (float)f1.fb[0][0];
+        if (v == 12345.678f) g.out[t] = (half_t)v;
+        return;
+    }
     nt_epilogue<TM, TN, WM, WN>(g, acc, smem, s, i0, j0, wi, wj, wave, lane);
 }
 
@@ -1074,3 +1097,16 @@ hipError_t launch_gemm_nt(const Problem &p0, const void *A, const void *B, const
 }
 
 } // namespace rt
+
+#if RT_NT_ABLATION
+// Entry point of a timing-only build of this file (see RT_NT_ABLATION): the Linear form W[n x k] . X[m x k]^T + bias
+// with f16 weights, output [m x n].  The measurement probes library holds one such build per variant.
+extern "C" __attribute__((visibility("default"))) int RT_NT_ABL_ENTRY(const void *W, const void *X, const void *bias, void *out,
+                                                                      int64_t n, int64_t m, int64_t k, void *stream) {
+    rt::Problem p;
+    p.a_dt = RT_F16, p.act_dt = RT_F16, p.M = n, p.N = m, p.K = k;
+    p.a_rs = k, p.a_ks = 1, p.b_ks = 1, p.b_js = k, p.o_is = 1, p.o_js = n, p.has_bias = true, p.bias_on_rows = true;
+    p.kernel = RT_KERNEL_GEMM_F16;
+    return (int)rt::launch_gemm_nt(p, W, X, bias, out, (hipStream_t)stream, rt::DeviceInfo{});
+}
+#endif
