@@ -323,7 +323,9 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
         if ((st = check_extent(ctx, lhs, nl, "lhs")) != RT_OK || (st = check_extent(ctx, rhs, nr, "rhs")) != RT_OK ||
             (st = check_extent(ctx, desc->has_bias ? bias : nullptr, nb, "bias")) != RT_OK ||
             (st = check_extent(ctx, out, no, "out")) != RT_OK ||
-            (st = check_extent(ctx, p.workspace, p.workspace_bytes, "workspace")) != RT_OK)
+            // the library's own static scratch is a device symbol of known size, not an allocation to look up
+            (p.workspace != ctx->static_scratch &&
+             (st = check_extent(ctx, p.workspace, p.workspace_bytes, "workspace")) != RT_OK))
             return st;
     }
     hipError_t e = hipErrorNotSupported;
@@ -362,6 +364,7 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
 rt_status rt_matmul_enqueue_static(rt_ctx *ctx, const rt_matmul_desc *desc, const void *lhs, const void *rhs,
                                    const void *bias, void *out, int32_t activation, void *stream) {
     if (!ctx || !desc) return RT_ERR_INVALID_ARG;
+    RT_GUARD_BEGIN
     uint64_t need = 0;
     const rt_status st = rt_matmul_workspace_bytes(ctx, desc, &need);
     if (st != RT_OK) return st;
@@ -375,6 +378,7 @@ rt_status rt_matmul_enqueue_static(rt_ctx *ctx, const rt_matmul_desc *desc, cons
         return hip_fail(ctx, "rt_matmul_enqueue_static: hipGetSymbolAddress of the static scratch failed", ctx->static_scratch_err);
     // every share's sums are written before the second kernel reads them, so nothing needs clearing
     return rt_matmul_enqueue_ws(ctx, desc, lhs, rhs, bias, out, activation, ctx->static_scratch, kStaticScratchBytes, stream);
+    RT_GUARD_END(ctx)
 }
 
 rt_status rt_quantize_q8_0(rt_ctx *ctx, const void *src_f32, uint64_t numel, void *dst, void *stream) {

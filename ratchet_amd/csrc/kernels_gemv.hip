@@ -337,7 +337,9 @@ hipError_t launch_gemv(const Problem &p, const void *A, const void *B, const voi
         // at 5 / 7 / 8 vectors here); the conditions are the ones under which it takes the product
         if (p.a_dt == RT_F16 && p.act_dt == RT_F16 && p.N >= 5 && p.stacks == 1 && p.K > 256 && p.K % 64 == 0 &&
             (p.M + 63) / 64 >= dev.num_cus / 2 && p.a_ks == 1 && p.b_ks == 1 && aligned16(A) && aligned16(B) &&
-            (p.a_rs * 2) % 16 == 0 && (p.b_js * 2) % 16 == 0)
+            (p.a_rs * 2) % 16 == 0 && (p.b_js * 2) % 16 == 0 && !(p.o_js == 1 && p.o_is != 1))
+            // (a row-major output would make the tiled kernel exchange the operands, and with the weight as its
+            // activation side it declines: such a product stays here)
             return hipErrorNotSupported;
     }
     if (p.N < 1 || p.N > kGemvMaxCols || p.stacks > 65535) return hipErrorNotSupported;

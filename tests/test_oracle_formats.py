@@ -224,8 +224,7 @@ def test_q4k_known_answer_block(oracle, q4k_kat):
         assert oracle.q4k_scale_min(j, blk[4:16]) == scmn[j]
     assert np.array_equal(oracle.q4k_dequantize(blk).view(np.uint32), want.view(np.uint32))
     # and the packer used by the other tests agrees with the hand-typed bytes
-    nib = np.concatenate([np.array(n + n) for _, _, n in __import__("conftest").Q4K_KAT_SUBBLOCKS])
-    assert np.array_equal(_q4k_block(0.375, 0.625, [s for s, _ in scmn], [m for _, m in scmn], nib), blk)
+    assert np.array_equal(_q4k_block(q4k_kat.d, q4k_kat.dmin, [s for s, _ in scmn], [m for _, m in scmn], q4k_kat.nibbles), blk)
 
 
 def test_q4k_quantizer_round_trip(oracle):

@@ -89,3 +89,47 @@ def test_static_scratch_unsplit_product_and_errors(device, oracle):
     assert L.rt_matmul_enqueue_static(device.ctx, ctypes.byref(bad), dw.data_ptr(), dx.data_ptr(), None,
                                       ctypes.c_void_p(dx.data_ptr()), _ffi.RT_ACT_NONE, stream) == _ffi.RT_ERR_INVALID_SHAPE
     assert L.rt_matmul_enqueue_static(None, ctypes.byref(desc), None, None, None, None, 0, None) == _ffi.RT_ERR_INVALID_ARG
+
+
+def test_static_scratch_allocates_nothing_and_passes_checked_mode(device, oracle, monkeypatch):
+    """What the entry point exists for: device memory in use is the same before and after its calls; the buffer
+    holds what the Phi-2 prefill down-projection's split asks for; and in checked mode (RATCHET_CHECKED) the library
+    does not look its own static buffer up as if it were a caller's allocation."""
+    L = _ffi.lib()
+    N, M, K = 2560, 512, 10240
+    desc = _ffi.make_desc(_ffi.RT_Q8_0H, (N, K), _ffi.RT_F16, (1, M, K), False, True, True, _ffi.RT_F16, (N,))
+    need = ctypes.c_uint64()
+    assert L.rt_matmul_workspace_bytes(device.ctx, ctypes.byref(desc), ctypes.byref(need)) == _ffi.RT_OK
+    static_bytes = 20 << 20   # RT_STATIC_SCRATCH_BYTES of include/ratchet_hip.h
+    assert 0 < need.value <= static_bytes
+    rng = np.random.default_rng(4)
+    wbuf = oracle.make_q8_0h((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    x = rng.standard_normal((1, M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    dw, dx, db = _dev(wbuf), _dev(x), _dev(bias)
+    out = torch.empty(M * N * 2, dtype=torch.uint8, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call(ctx):
+        return L.rt_matmul_enqueue_static(ctx, ctypes.byref(desc), dw.data_ptr(), dx.data_ptr(), db.data_ptr(),
+                                          ctypes.c_void_p(out.data_ptr()), _ffi.RT_ACT_NONE, stream)
+    assert call(device.ctx) == _ffi.RT_OK   # warm-up: code objects loaded, kernel attributes set
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert call(device.ctx) == _ffi.RT_OK
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    first = out.cpu().numpy().copy()
+    # checked mode: a context created with RATCHET_CHECKED set runs the same call
+    monkeypatch.setenv("RATCHET_CHECKED", "1")
+    ctx = ctypes.c_void_p()
+    assert L.rt_ctx_create(device.ordinal, ctypes.byref(ctx)) == _ffi.RT_OK
+    try:
+        out.fill_(0xEE)
+        assert call(ctx) == _ffi.RT_OK, L.rt_last_error(ctx)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), first)
+    finally:
+        L.rt_ctx_destroy(ctx)
