@@ -764,6 +764,44 @@ def issue_calibration(r: Runner):
     return {"issue_calibration": rows, "trips": iters, "wavefronts_per_simd": 1}
 
 
+def host_enqueue_cost(r: Runner, O, calls=2000):
+    """Host microseconds per enqueue of the headline GEMV through rt_matmul_enqueue_ws (guards, shape rules and
+    lowering on every call) and through a plan (rt_matmul_plan_create once, rt_matmul_plan_enqueue per call): `calls`
+    back-to-back calls from a C++ loop in ratchet_amd/libratchet_probes.so, host steady clock, no Python in the loop."""
+    N, K = 10240, 2560
+    rng = np.random.default_rng(0)
+    wd = r.upload(O.make_q8_0h((rng.standard_normal((N, K)) * 0.02).astype(np.float32)))
+    xd, bd = r.upload(rng.standard_normal((1, 1, K)).astype(np.float16)), r.upload(rng.standard_normal(N).astype(np.float16))
+    out = r.torch.empty(N * 2, dtype=r.torch.uint8, device="cuda:0")
+    desc = r.ffi.make_desc(r.ffi.RT_Q8_0H, (N, K), r.ffi.RT_F16, (1, 1, K), False, True, True, r.ffi.RT_F16, (N,))
+    P = ctypes.CDLL(os.path.join(ROOT, "ratchet_amd", "libratchet_probes.so"))
+    vp = ctypes.c_void_p
+    P.probe_host_ns_enqueue_ws.restype = P.probe_host_ns_plan_enqueue.restype = ctypes.c_double
+    P.probe_host_ns_enqueue_ws.argtypes = [vp, vp, vp, vp, vp, vp, vp, ctypes.c_int32, vp, ctypes.c_int]
+    P.probe_host_ns_plan_enqueue.argtypes = [vp, vp, vp, vp, vp, vp, vp, ctypes.c_int]
+    addr = lambda name: ctypes.cast(getattr(r.L, name), vp)
+    stream = vp(r.torch.cuda.current_stream().cuda_stream)
+    plan = vp()
+    if r.L.rt_matmul_plan_create(r.dev.ctx, ctypes.byref(desc), 0, ctypes.byref(plan)) != r.ffi.RT_OK:
+        raise RuntimeError("rt_matmul_plan_create failed")
+    res = {}
+    try:
+        for _ in range(2):  # the first pass warms the code paths
+            a = P.probe_host_ns_enqueue_ws(addr("rt_matmul_enqueue_ws"), r.dev.ctx, ctypes.byref(desc), vp(wd.data_ptr()), vp(xd.data_ptr()),
+                                           vp(bd.data_ptr()), vp(out.data_ptr()), 0, stream, calls)
+            r.torch.cuda.synchronize()
+            b = P.probe_host_ns_plan_enqueue(addr("rt_matmul_plan_enqueue"), plan, vp(wd.data_ptr()), vp(xd.data_ptr()), vp(bd.data_ptr()),
+                                             vp(out.data_ptr()), stream, calls)
+            r.torch.cuda.synchronize()
+        if a < 0 or b < 0:
+            raise RuntimeError("an enqueue failed inside the host-cost probe")
+        res = {"rt_matmul_enqueue_ws": round(a * 1e-3, 3), "rt_matmul_plan_enqueue": round(b * 1e-3, 3), "calls": calls,
+               "how": "back-to-back calls from a C++ loop (no Python), host steady clock, launches piling up on the stream"}
+    finally:
+        r.L.rt_matmul_plan_destroy(plan)
+    return res
+
+
 def gemm_ablation(r: Runner):
     """What bounds the f16 tiled GEMM at X[512 x 2560] . W[10240 x 2560]^T + bias: the shipped kernel next to timing-only
     builds of the same source with parts left out (their results are wrong; ratchet_amd/libratchet_probes.so holds them,
@@ -960,6 +998,7 @@ def main():
             # no HIP event involved: host clock around 2000 replays of a graph of one rotation, between two synchronisations
             "wall_clock_ms_per_step": head["stats"]["wall_clock_ms_per_step"],
             "wall_clock_launches": head["stats"]["wall_clock_launches"],
+            "host_us_per_enqueue": host_enqueue_cost(r, O),
         },
         "roofline": {
             "bound": "hbm",

@@ -126,6 +126,10 @@ pub struct rt_ctx {
 pub struct rt_gguf {
     _private: [u8; 0],
 }
+#[repr(C)]
+pub struct rt_matmul_plan {
+    _private: [u8; 0],
+}
 
 #[link(name = "ratchet_hip")]
 extern "C" {
@@ -158,6 +162,11 @@ extern "C" {
                                 workspace_bytes: u64, stream: *mut c_void) -> rt_status;
     pub fn rt_matmul_enqueue_static(ctx: *mut rt_ctx, d: *const rt_matmul_desc, lhs: *const c_void, rhs: *const c_void,
                                     bias: *const c_void, out: *mut c_void, activation: i32, stream: *mut c_void) -> rt_status;
+    // the operator, compiled once: guards, shape rules and lowering at creation; an enqueue takes pointers only
+    pub fn rt_matmul_plan_create(ctx: *mut rt_ctx, d: *const rt_matmul_desc, activation: i32, plan: *mut *mut rt_matmul_plan) -> rt_status;
+    pub fn rt_matmul_plan_enqueue(plan: *mut rt_matmul_plan, lhs: *const c_void, rhs: *const c_void, bias: *const c_void,
+                                  out: *mut c_void, workspace: *mut c_void, workspace_bytes: u64, stream: *mut c_void) -> rt_status;
+    pub fn rt_matmul_plan_destroy(plan: *mut rt_matmul_plan) -> rt_status;
     // block formats on the device
     pub fn rt_quantize_q8_0(ctx: *mut rt_ctx, src_f32: *const c_void, numel: u64, dst: *mut c_void, stream: *mut c_void) -> rt_status;
     pub fn rt_dequantize(ctx: *mut rt_ctx, dtype: i32, src: *const c_void, numel: u64, dst_f32: *mut c_void, stream: *mut c_void) -> rt_status;

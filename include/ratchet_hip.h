@@ -350,6 +350,22 @@ RT_API rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, c
 RT_API rt_status rt_matmul_enqueue_static(rt_ctx *ctx, const rt_matmul_desc *desc, const void *lhs, const void *rhs,
                                           const void *bias, void *out, int32_t activation, void *stream);
 
+/* The compile-once half of the operator.  In the reference an operator is compiled once per graph
+ * (Matmul::kernel_key names the pipeline, ops/matmul.rs:485-524; Operation::compile builds the
+ * CompiledOp with its workgroup count and bindings, op.rs:304-362) and Executable::dispatch_operations
+ * (executable.rs:25-54) only records the dispatch on every step.  A plan is that for this library:
+ * rt_matmul_plan_create runs the guards, the shape rules and the lowering of `desc` (what every
+ * rt_matmul_enqueue* call repeats) once and fixes the fused activation; rt_matmul_plan_enqueue takes only
+ * the device pointers (and a workspace as rt_matmul_enqueue_ws does, or NULL, 0), offers the product first
+ * to the kernel family that took it last time, and launches.  Results are those of rt_matmul_enqueue_ws with
+ * the same arguments, bit for bit (the same kernels run).  A plan belongs to the context it was created
+ * with, may be enqueued from several threads, and must be destroyed before that context. */
+typedef struct rt_matmul_plan rt_matmul_plan;
+RT_API rt_status rt_matmul_plan_create(rt_ctx *ctx, const rt_matmul_desc *desc, int32_t activation, rt_matmul_plan **plan);
+RT_API rt_status rt_matmul_plan_enqueue(rt_matmul_plan *plan, const void *lhs, const void *rhs, const void *bias,
+                                        void *out, void *workspace, uint64_t workspace_bytes, void *stream);
+RT_API rt_status rt_matmul_plan_destroy(rt_matmul_plan *plan);
+
 /* Replaces: Unary (ops/unary.rs:71-260) for Gelu and Silu on F32 / F16 tensors; `dst` may be
  * `src` (the reference runs unary operators in place when it can). */
 RT_API rt_status rt_unary_enqueue(rt_ctx *ctx, int32_t activation, int32_t dtype, const void *src, void *dst,

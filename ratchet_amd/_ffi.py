@@ -103,6 +103,9 @@ SIGNATURES = {
     "rt_matmul_workspace_bytes": (_i32, [_vp, _P(MatmulDesc), _P(_u64)]),
     "rt_matmul_enqueue_ws": (_i32, [_vp, _P(MatmulDesc), _vp, _vp, _vp, _vp, _i32, _vp, _u64, _vp]),
     "rt_matmul_enqueue_static": (_i32, [_vp, _P(MatmulDesc), _vp, _vp, _vp, _vp, _i32, _vp]),
+    "rt_matmul_plan_create": (_i32, [_vp, _P(MatmulDesc), _i32, _P(_vp)]),
+    "rt_matmul_plan_enqueue": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]),
+    "rt_matmul_plan_destroy": (_i32, [_vp]),
     "rt_unary_enqueue": (_i32, [_vp, _i32, _i32, _vp, _vp, _u64, _vp]),
     "rt_cast_enqueue": (_i32, [_vp, _i32, _i32, _vp, _vp, _u64, _vp]),
     "rt_quantize_q8_0": (_i32, [_vp, _vp, _u64, _vp, _vp]),

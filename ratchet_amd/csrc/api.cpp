@@ -3,8 +3,10 @@
 // host: a missing device is an error, never a fallback.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <new>
 #include <string>
@@ -101,7 +103,100 @@ struct DeviceGuard {
     catch (const std::exception &e) { return fail(ctx, RT_ERR_INVALID_ARG, e.what()); }            \
     catch (...) { return fail(ctx, RT_ERR_INVALID_ARG, "unknown exception"); }
 
+
+// A descriptor lowered once: the strided problem with its kernel family, and what checked mode compares
+// the operands' allocations with.
+struct Lowered {
+    rt::Problem p;
+    bool has_bias = false;
+    uint64_t lhs_bytes = 0, rhs_bytes = 0, bias_bytes = 0, out_bytes = 0;
+};
+
+rt_status lower_matmul(rt_ctx *ctx, const rt_matmul_desc &desc, int32_t activation, Lowered &low) {
+    if (activation != RT_ACT_NONE && activation != RT_ACT_GELU && activation != RT_ACT_SILU)
+        return fail(ctx, RT_ERR_INVALID_ARG, "unknown activation");
+    rt_gemm_spec spec;
+    std::string why;
+    const rt_status st = rt::make_spec(desc, spec, low.p, &why);
+    if (st != RT_OK) return fail(ctx, st, why);
+    low.p.act = activation;
+    low.has_bias = desc.has_bias != 0;
+    if (ctx->checked &&
+        (rt_tensor_nbytes(desc.lhs_dt, shape_numel(desc.lhs_shape, desc.lhs_rank), &low.lhs_bytes) != RT_OK ||
+         rt_tensor_nbytes(desc.rhs_dt, shape_numel(desc.rhs_shape, desc.rhs_rank), &low.rhs_bytes) != RT_OK ||
+         (desc.has_bias && rt_tensor_nbytes(desc.bias_dt, shape_numel(desc.bias_shape, desc.bias_rank), &low.bias_bytes) != RT_OK)))
+        return fail(ctx, RT_ERR_INVALID_ARG, "checked: operand sizes");
+    low.out_bytes = (uint64_t)low.p.stacks * (uint64_t)low.p.M * (uint64_t)low.p.N * (low.p.act_dt == RT_F16 ? 2u : 4u);
+    return RT_OK;
+}
+
+// The kernel families in the order they are offered a problem; each declines (hipErrorNotSupported) what it
+// does not take.  The first two see the streaming kernel kinds make_spec chose; from the third on the problem is
+// a tiled one.
+using Launcher = hipError_t (*)(const rt::Problem &, const void *, const void *, const void *, void *, hipStream_t,
+                                const rt::DeviceInfo &);
+constexpr Launcher kLaunchers[] = {rt::launch_gemv,          // streaming kernels
+                                   rt::launch_gemv_chunked,  // Q8_0H / Q4_K weights against a few vectors more than one streaming launch takes
+                                   rt::launch_gemm_nt,       // K-contiguous f16 / Q8_0H problems: the large-tile kernel
+                                   rt::launch_gemm_nn_smalln, // f16 products with an untransposed narrow rhs (attention P.V)
+                                   rt::launch_gemm_f32,      // f32 products whose operands each have a contiguous axis
+                                   rt::launch_gemm_q4k,      // Q4_K weights against many activation rows
+                                   rt::launch_gemm};         // anything
+constexpr int kNumLaunchers = (int)(sizeof(kLaunchers) / sizeof(kLaunchers[0])), kFirstTiled = 2;
+
+// `hint` (a plan's memory): the family that took this problem last time is offered it first.
+rt_status run_matmul(rt_ctx *ctx, const Lowered &low, const void *lhs, const void *rhs, const void *bias, void *out,
+                     void *workspace, uint64_t workspace_bytes, void *stream, std::atomic<int> *hint) {
+    rt::Problem p = low.p;
+    p.workspace = workspace_bytes ? workspace : nullptr, p.workspace_bytes = workspace ? workspace_bytes : 0;
+    if (p.kernel == RT_KERNEL_NONE) return RT_OK; // empty output
+    if (!lhs || !rhs || !out || (low.has_bias && !bias)) return fail(ctx, RT_ERR_INVALID_ARG, "null device pointer");
+    const void *A = p.swapped ? rhs : lhs, *B = p.swapped ? lhs : rhs;
+    const void *bp = low.has_bias ? bias : nullptr;
+    DeviceGuard dg(ctx->dev.ordinal);
+    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
+    if (ctx->checked) {
+        rt_status st;
+        if ((st = check_extent(ctx, lhs, low.lhs_bytes, "lhs")) != RT_OK || (st = check_extent(ctx, rhs, low.rhs_bytes, "rhs")) != RT_OK ||
+            (st = check_extent(ctx, bp, low.bias_bytes, "bias")) != RT_OK || (st = check_extent(ctx, out, low.out_bytes, "out")) != RT_OK ||
+            // the library's own static scratch is a device symbol of known size, not an allocation to look up
+            (p.workspace != ctx->static_scratch &&
+             (st = check_extent(ctx, p.workspace, p.workspace_bytes, "workspace")) != RT_OK))
+            return st;
+    }
+    const bool streaming = p.kernel == RT_KERNEL_GEMV_Q8 || p.kernel == RT_KERNEL_GEMV_Q4K || p.kernel == RT_KERNEL_GEMV_FLOAT;
+    const int tiled_kind = p.act_dt == RT_F16 ? RT_KERNEL_GEMM_F16 : RT_KERNEL_GEMM_F32;
+    hipError_t e = hipErrorNotSupported;
+    const int first = hint ? hint->load(std::memory_order_relaxed) : -1;
+    if (first >= 0) {
+        if (first >= kFirstTiled) p.kernel = tiled_kind;
+        e = kLaunchers[first](p, A, B, bp, out, (hipStream_t)stream, ctx->dev);
+        if (e == hipErrorNotSupported) p.kernel = low.p.kernel; // other pointers than last time: ask everyone again
+    }
+    for (int i = streaming ? 0 : 1; i < kNumLaunchers && e == hipErrorNotSupported; i++) {
+        if (i == first) continue;
+        // operands that miss the streaming kernels' alignment take the tiled kernels
+        if (i >= kFirstTiled) p.kernel = tiled_kind;
+        e = kLaunchers[i](p, A, B, bp, out, (hipStream_t)stream, ctx->dev);
+        if (e == hipSuccess && hint) hint->store(i, std::memory_order_relaxed);
+    }
+    // no kernel takes the shape (more than 65535 stacks or row tiles of the generic kernel, a misaligned
+    // quantized operand): a limit of this library, not a failure of the runtime
+    if (e == hipErrorNotSupported)
+        return fail(ctx, RT_ERR_UNSUPPORTED, "matmul: no kernel takes this shape (over 65535 stacks or 65535 row tiles, or a "
+                                             "quantized operand that is not 16-byte aligned)");
+    if (e != hipSuccess) return hip_fail(ctx, "matmul launch", e);
+    return RT_OK;
+}
+
 } // namespace
+
+// What rt_matmul_plan_create keeps: the lowered problem, and which kernel family took it last time.
+struct rt_matmul_plan {
+    rt_ctx *ctx = nullptr;
+    Lowered low;
+    std::atomic<int> launcher{-1};
+};
 
 extern "C" {
 
@@ -298,67 +393,37 @@ rt_status rt_matmul_enqueue_ws(rt_ctx *ctx, const rt_matmul_desc *desc, const vo
                                uint64_t workspace_bytes, void *stream) {
     if (!ctx || !desc) return RT_ERR_INVALID_ARG;
     RT_GUARD_BEGIN
-    if (activation != RT_ACT_NONE && activation != RT_ACT_GELU && activation != RT_ACT_SILU)
-        return fail(ctx, RT_ERR_INVALID_ARG, "unknown activation");
-    rt_gemm_spec spec;
-    rt::Problem p;
-    std::string why;
-    rt_status st = rt::make_spec(*desc, spec, p, &why);
-    if (st != RT_OK) return fail(ctx, st, why);
-    p.act = activation;
-    p.workspace = workspace_bytes ? workspace : nullptr, p.workspace_bytes = workspace ? workspace_bytes : 0;
-    if (p.kernel == RT_KERNEL_NONE) return RT_OK; // empty output
-    if (!lhs || !rhs || !out || (desc->has_bias && !bias))
-        return fail(ctx, RT_ERR_INVALID_ARG, "null device pointer");
-    const void *A = p.swapped ? rhs : lhs, *B = p.swapped ? lhs : rhs;
-    DeviceGuard dg(ctx->dev.ordinal);
-    if (!dg.ok) return fail(ctx, RT_ERR_NO_DEVICE, "hipSetDevice failed");
-    if (ctx->checked) {
-        uint64_t nl = 0, nr = 0, nb = 0;
-        if (rt_tensor_nbytes(desc->lhs_dt, shape_numel(desc->lhs_shape, desc->lhs_rank), &nl) != RT_OK ||
-            rt_tensor_nbytes(desc->rhs_dt, shape_numel(desc->rhs_shape, desc->rhs_rank), &nr) != RT_OK ||
-            (desc->has_bias && rt_tensor_nbytes(desc->bias_dt, shape_numel(desc->bias_shape, desc->bias_rank), &nb) != RT_OK))
-            return fail(ctx, RT_ERR_INVALID_ARG, "checked: operand sizes");
-        const uint64_t no = (uint64_t)p.stacks * (uint64_t)p.M * (uint64_t)p.N * (p.act_dt == RT_F16 ? 2u : 4u);
-        if ((st = check_extent(ctx, lhs, nl, "lhs")) != RT_OK || (st = check_extent(ctx, rhs, nr, "rhs")) != RT_OK ||
-            (st = check_extent(ctx, desc->has_bias ? bias : nullptr, nb, "bias")) != RT_OK ||
-            (st = check_extent(ctx, out, no, "out")) != RT_OK ||
-            // the library's own static scratch is a device symbol of known size, not an allocation to look up
-            (p.workspace != ctx->static_scratch &&
-             (st = check_extent(ctx, p.workspace, p.workspace_bytes, "workspace")) != RT_OK))
-            return st;
-    }
-    hipError_t e = hipErrorNotSupported;
-    if (p.kernel == RT_KERNEL_GEMV_Q8 || p.kernel == RT_KERNEL_GEMV_Q4K || p.kernel == RT_KERNEL_GEMV_FLOAT)
-        e = rt::launch_gemv(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-    // Q8_0H / Q4_K weights against a few vectors more than one streaming launch takes: one launch per 16
-    if (e == hipErrorNotSupported)
-        e = rt::launch_gemv_chunked(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-    if (e == hipErrorNotSupported) {
-        // operands that miss the streaming kernels' alignment take the tiled GEMM
-        p.kernel = p.act_dt == RT_F16 ? RT_KERNEL_GEMM_F16 : RT_KERNEL_GEMM_F32;
-        // K-contiguous f16 / Q8_0H problems: the large-tile kernel; it declines what it cannot take
-        e = rt::launch_gemm_nt(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-        // f16 products with an untransposed narrow rhs (attention P.V)
-        if (e == hipErrorNotSupported)
-            e = rt::launch_gemm_nn_smalln(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-        // f32 products whose operands each have a contiguous axis
-        if (e == hipErrorNotSupported)
-            e = rt::launch_gemm_f32(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-        // Q4_K weights against many activation rows
-        if (e == hipErrorNotSupported)
-            e = rt::launch_gemm_q4k(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-        if (e == hipErrorNotSupported)
-            e = rt::launch_gemm(p, A, B, desc->has_bias ? bias : nullptr, out, (hipStream_t)stream, ctx->dev);
-    }
-    // no kernel takes the shape (more than 65535 stacks or row tiles of the generic kernel, a misaligned
-    // quantized operand): a limit of this library, not a failure of the runtime
-    if (e == hipErrorNotSupported)
-        return fail(ctx, RT_ERR_UNSUPPORTED, "matmul: no kernel takes this shape (over 65535 stacks or 65535 row tiles, or a "
-                                             "quantized operand that is not 16-byte aligned)");
-    if (e != hipSuccess) return hip_fail(ctx, "matmul launch", e);
+    Lowered low;
+    const rt_status st = lower_matmul(ctx, *desc, activation, low);
+    if (st != RT_OK) return st;
+    return run_matmul(ctx, low, lhs, rhs, bias, out, workspace, workspace_bytes, stream, nullptr);
+    RT_GUARD_END(ctx)
+}
+
+rt_status rt_matmul_plan_create(rt_ctx *ctx, const rt_matmul_desc *desc, int32_t activation, rt_matmul_plan **plan) {
+    if (!ctx || !desc || !plan) return RT_ERR_INVALID_ARG;
+    *plan = nullptr;
+    RT_GUARD_BEGIN
+    std::unique_ptr<rt_matmul_plan> pl(new rt_matmul_plan);
+    pl->ctx = ctx;
+    const rt_status st = lower_matmul(ctx, *desc, activation, pl->low);
+    if (st != RT_OK) return st;
+    *plan = pl.release();
     return RT_OK;
     RT_GUARD_END(ctx)
+}
+
+rt_status rt_matmul_plan_enqueue(rt_matmul_plan *plan, const void *lhs, const void *rhs, const void *bias, void *out,
+                                 void *workspace, uint64_t workspace_bytes, void *stream) {
+    if (!plan) return RT_ERR_INVALID_ARG;
+    RT_GUARD_BEGIN
+    return run_matmul(plan->ctx, plan->low, lhs, rhs, bias, out, workspace, workspace_bytes, stream, &plan->launcher);
+    RT_GUARD_END(plan->ctx)
+}
+
+rt_status rt_matmul_plan_destroy(rt_matmul_plan *plan) {
+    delete plan;
+    return RT_OK;
 }
 
 rt_status rt_matmul_enqueue_static(rt_ctx *ctx, const rt_matmul_desc *desc, const void *lhs, const void *rhs,

@@ -6,6 +6,7 @@
 // libratchet_probes.so; the product library does not contain them and nothing else uses them.
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cstdint>
 
 typedef uint32_t probe_u4 __attribute__((ext_vector_type(4)));
@@ -164,5 +165,30 @@ __attribute__((visibility("default"))) int probe_read_rows16(const void *p, int6
     hipLaunchKernelGGL(probe_read_rows16_kernel, dim3((unsigned)(rows / 16)), dim3((unsigned)(K / 256) * 64), 0,
                        (hipStream_t)stream, (const uint8_t *)p, K, (uint32_t *)sink);
     return (int)hipGetLastError();
+}
+
+// What the host spends per enqueue, with no interpreter in the loop: n back-to-back calls of the entry point whose
+// address is `fn` (rt_matmul_enqueue_ws or rt_matmul_plan_enqueue of the product library, handed over by the
+// caller so that this library does not link against it), timed with the host's steady clock.  The launches pile up
+// on the stream; the caller synchronises afterwards.  Returns nanoseconds per call, or -1 if a call failed.
+__attribute__((visibility("default"))) double probe_host_ns_enqueue_ws(void *fn, void *ctx, const void *desc, const void *lhs,
+                                                                       const void *rhs, const void *bias, void *out,
+                                                                       int32_t act, void *stream, int n) {
+    typedef int32_t (*F)(void *, const void *, const void *, const void *, const void *, void *, int32_t, void *, uint64_t, void *);
+    const F f = (F)fn;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < n; i++)
+        if (f(ctx, desc, lhs, rhs, bias, out, act, nullptr, 0, stream) != 0) return -1.0;
+    return std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count() / n;
+}
+
+__attribute__((visibility("default"))) double probe_host_ns_plan_enqueue(void *fn, void *plan, const void *lhs, const void *rhs,
+                                                                         const void *bias, void *out, void *stream, int n) {
+    typedef int32_t (*F)(void *, const void *, const void *, const void *, void *, void *, uint64_t, void *);
+    const F f = (F)fn;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < n; i++)
+        if (f(plan, lhs, rhs, bias, out, nullptr, 0, stream) != 0) return -1.0;
+    return std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count() / n;
 }
 }

@@ -203,3 +203,68 @@ def test_f16_weight_beyond_2_31_elements(device, oracle):
     got = Tensor.from_data(w).to(device).gemm(Tensor.from_data(x).to(device), None, False, True, True).resolve()
     got = got.to(Device.CPU).storage                                    # [1, M, N]
     assert np.array_equal(got[0], w[:, cols].T)
+
+
+def test_plan_enqueue_equals_plain_enqueue_on_the_five_configs(device, oracle):
+    """rt_matmul_plan_create + rt_matmul_plan_enqueue against rt_matmul_enqueue_ws on the BASELINE shapes (C1, C2 at
+    1 / 4 / 8 vectors, both C3 products, C4 up and down with a workspace, C5 at 1 / 16 / 256 rows): the same kernels
+    run, so the outputs agree bit for bit, on the first enqueue of a plan (which asks every kernel family in turn)
+    and on the second (which goes straight to the one that took it)."""
+    import ctypes
+
+    import torch
+
+    from ratchet_amd import _ffi
+    L = _ffi.lib()
+    rng = np.random.default_rng(50)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1).copy()).cuda()
+    f16 = lambda *s: rng.standard_normal(s).astype(np.float16)
+    q8 = lambda n, k: oracle.make_q8_0h((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    q4 = lambda n, k: oracle.q4k_quantize((rng.standard_normal(n * k) * 0.02).astype(np.float32))
+    F32, F16, Q8, Q4 = _ffi.RT_F32, _ffi.RT_F16, _ffi.RT_Q8_0H, _ffi.RT_Q4_K
+    cases = [  # (lhs, dtype, shape, rhs, dtype, shape, bias, trans flags, output bytes)
+        ((rng.standard_normal((1500, 384)) * 0.05).astype(np.float32), F32, (1500, 384),
+         (rng.standard_normal((384, 1536)) * 0.05).astype(np.float32), F32, (384, 1536),
+         (rng.standard_normal(1536) * 0.05).astype(np.float32), (False, False, False), 1500 * 1536 * 4)]
+    w_up = q8(10240, 2560)
+    for m in (1, 4, 8, 512):
+        cases.append((w_up, Q8, (10240, 2560), f16(1, m, 2560), F16, (1, m, 2560), f16(10240), (False, True, True), m * 10240 * 2))
+    cases.append((q8(2560, 10240), Q8, (2560, 10240), f16(1, 512, 10240), F16, (1, 512, 10240), f16(2560), (False, True, True), 512 * 2560 * 2))
+    cases.append((f16(1, 32, 512, 80), F16, (1, 32, 512, 80), f16(1, 32, 512, 80), F16, (1, 32, 512, 80), None, (False, True, False), 32 * 512 * 512 * 2))
+    cases.append(((rng.random((1, 32, 512, 512)) / 512).astype(np.float16), F16, (1, 32, 512, 512), f16(1, 32, 512, 80), F16,
+                  (1, 32, 512, 80), None, (False, False, False), 32 * 512 * 80 * 2))
+    w_q4 = q4(8192, 3072)
+    for m in (1, 16, 256):
+        cases.append((w_q4, Q4, (8192, 3072), f16(1, m, 3072), F16, (1, m, 3072), None, (False, True, True), m * 8192 * 2))
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for i, (lhs, ldt, lshape, rhs, rdt, rshape, bias, flags, out_bytes) in enumerate(cases):
+        desc = (_ffi.make_desc(ldt, lshape, rdt, rshape, *flags) if bias is None else
+                _ffi.make_desc(ldt, lshape, rdt, rshape, *flags, F16 if bias.dtype == np.float16 else F32, bias.shape))
+        dl, dr, db = dev(lhs), dev(rhs), None if bias is None else dev(bias)
+        bp = None if db is None else ctypes.c_void_p(db.data_ptr())
+        need = ctypes.c_uint64()
+        assert L.rt_matmul_workspace_bytes(device.ctx, ctypes.byref(desc), ctypes.byref(need)) == _ffi.RT_OK
+        ws = torch.empty(need.value, dtype=torch.uint8, device="cuda") if need.value else None
+        wp = None if ws is None else ctypes.c_void_p(ws.data_ptr())
+        outs = [torch.full((out_bytes,), 0xEE, dtype=torch.uint8, device="cuda") for _ in range(3)]
+        st = L.rt_matmul_enqueue_ws(device.ctx, ctypes.byref(desc), dl.data_ptr(), dr.data_ptr(), bp,
+                                    ctypes.c_void_p(outs[0].data_ptr()), 0, wp, need.value, stream)
+        assert st == _ffi.RT_OK, (i, L.rt_last_error(device.ctx))
+        plan = ctypes.c_void_p()
+        assert L.rt_matmul_plan_create(device.ctx, ctypes.byref(desc), 0, ctypes.byref(plan)) == _ffi.RT_OK, i
+        try:
+            for o in outs[1:]:
+                st = L.rt_matmul_plan_enqueue(plan, dl.data_ptr(), dr.data_ptr(), bp, ctypes.c_void_p(o.data_ptr()), wp, need.value, stream)
+                assert st == _ffi.RT_OK, (i, L.rt_last_error(device.ctx))
+            torch.cuda.synchronize()
+        finally:
+            L.rt_matmul_plan_destroy(plan)
+        a = outs[0].cpu().numpy()
+        assert not np.all(a == 0xEE)
+        assert np.array_equal(a, outs[1].cpu().numpy()) and np.array_equal(a, outs[2].cpu().numpy()), i
+    # descriptor errors surface when the plan is created; a null plan is a status
+    bad = _ffi.make_desc(F16, (64, 32), F16, (1, 8, 40), False, True, True)
+    plan = ctypes.c_void_p()
+    assert L.rt_matmul_plan_create(device.ctx, ctypes.byref(bad), 0, ctypes.byref(plan)) == _ffi.RT_ERR_INVALID_SHAPE and not plan.value
+    assert L.rt_matmul_plan_create(device.ctx, ctypes.byref(bad), 99, ctypes.byref(plan)) == _ffi.RT_ERR_INVALID_ARG
+    assert L.rt_matmul_plan_enqueue(None, None, None, None, None, None, 0, None) == _ffi.RT_ERR_INVALID_ARG
