@@ -39,7 +39,10 @@ INFINITY_CACHE_BYTES = 256 << 20
 # HBM bytes per launch of the GEMV kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy); the commands and
 # readings are in profiles/gemv_q8_phi2_m1_pmc.txt.  A counter reading cannot be taken inside
-# this script, so the figure is the recorded one for the M=1 workload.
+# this script, so the figure is the recorded one for the M=1 workload.  The readings were taken on
+# the build whose gemv_q8h_rowdot_kernel / gemm_nt_dl_kernel sources are the ones in this tree
+# (git log -- ratchet_amd/csrc/kernels_gemv.hip ratchet_amd/csrc/kernels_gemm_nt.hip names the
+# last change to each); a change to either kernel's loads or stores needs the two --pmc runs again.
 GEMV_TRAFFIC_BYTES = 27985470
 # The same for the f16 GEMM of the metric's second half (profiles/gemm_c4_f16_q8_pmc.txt): FETCH_SIZE
 # 36,025 KiB x 1.99982 (copy calibration) + WRITE_SIZE 11,531 KiB.  The weight is read once and the
