@@ -26,7 +26,7 @@ NT_ABLATIONS = (4, 7, 8, 9, 13, 14, 15)
 
 SOURCES = ["api.cpp", "spec.cpp", "gguf.cpp", "kernels_blocks.hip", "kernels_softmax.hip", "kernels_unary.hip", "kernels_attention.hip", "kernels_gemv.hip", "kernels_gemv_mfma.hip", "kernels_gemv_rowdot.hip", "kernels_gemv_quad.hip", "kernels_gemv_rowfloat.hip",
     "kernels_gemv_q4k_mfma.hip", "kernels_gemv_q4k_rowdot.hip", "kernels_gemm.hip", "kernels_gemm_f32.hip", "kernels_gemm_q4k.hip",
-    "kernels_gemm_nt.hip", "kernels_gemm_nn.hip"]
+    "kernels_gemm_nt.hip", "kernels_gemm_nn.hip", "kernels_gemm_stream.hip"]
 HEADERS = ["spec.h", "device_common.h", os.path.join("..", "..", "include", "ratchet_hip.h")]
 
 # -packed-fp32-ops is switched off on purpose: the compiler then never forms

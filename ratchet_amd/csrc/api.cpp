@@ -137,6 +137,7 @@ using Launcher = hipError_t (*)(const rt::Problem &, const void *, const void *,
                                 const rt::DeviceInfo &);
 constexpr Launcher kLaunchers[] = {rt::launch_gemv,          // streaming kernels
                                    rt::launch_gemv_chunked,  // Q8_0H / Q4_K weights against a few vectors more than one streaming launch takes
+                                   rt::launch_gemm_stream,   // f16 / Q8_0H weights against a few dozen activation rows: one pass over the weight
                                    rt::launch_gemm_nt,       // K-contiguous f16 / Q8_0H problems: the large-tile kernel
                                    rt::launch_gemm_nn_smalln, // f16 products with an untransposed narrow rhs (attention P.V)
                                    rt::launch_gemm_f32,      // f32 products whose operands each have a contiguous axis

@@ -166,6 +166,8 @@ hipError_t launch_gemm_f32(const Problem &p, const void *A, const void *B, const
                            const DeviceInfo &dev);
 hipError_t launch_gemm(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                        hipStream_t stream, const DeviceInfo &dev);
+hipError_t launch_gemm_stream(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
+                              const DeviceInfo &dev);
 uint64_t gemm_nt_workspace_bytes(const Problem &p, const DeviceInfo &dev);
 hipError_t launch_gemm_nt(const Problem &p, const void *A, const void *B, const void *bias, void *out,
                           hipStream_t stream, const DeviceInfo &dev);

@@ -333,8 +333,9 @@ hipError_t launch_gemv(const Problem &p, const void *A, const void *B, const voi
         hipError_t e = launch_gemv_float_rowdot(p, A, B, bias, out, stream, dev);
         if (e != hipErrorNotSupported) return e;
         // 5..8 vectors against an f16 weight with enough rows that 64-row tiles give half of the compute units a
-        // workgroup: the tiled kernel's 64 x 64 tiles (10240 x 2560, weights from HBM: 16 us against 19 / 24 / 26 us
-        // at 5 / 7 / 8 vectors here); the conditions are the ones under which it takes the product
+        // workgroup: the weight-streaming GEMM, or the tiled kernel's 64 x 64 tiles (10240 x 2560, weights from HBM:
+        // 12.7 / 16 us against 19 / 24 / 26 us at 5 / 7 / 8 vectors here); the conditions are the ones under which
+        // the tiled kernel takes the product
         if (p.a_dt == RT_F16 && p.act_dt == RT_F16 && p.N >= 5 && p.stacks == 1 && p.K > 256 && p.K % 64 == 0 &&
             (p.M + 63) / 64 >= dev.num_cus / 2 && p.a_ks == 1 && p.b_ks == 1 && aligned16(A) && aligned16(B) &&
             (p.a_rs * 2) % 16 == 0 && (p.b_js * 2) % 16 == 0 && !(p.o_js == 1 && p.o_is != 1))

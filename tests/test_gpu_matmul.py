@@ -739,6 +739,64 @@ def test_f16_weights_few_activation_rows(device, oracle):
             check(oracle, got, want, DType.F16, (M, N, K, to))
 
 
+def test_weight_streaming_short_prompts(device, oracle):
+    """f16 weights against 5..64 and Q8_0H weights against 17..32 activation rows, K a multiple of 256 and enough
+    weight rows for three quarters of the compute units, take the weight-streaming GEMM: every tile count of
+    activation rows (and counts off the 16 of a tile), one to three tiles of weight rows per workgroup, row counts
+    off the 8 of a share (the scalar output path) and off the 16 of a tile, K from one step per wavefront (256) to
+    more steps than the register ring holds, the bias along the weight rows (trans_out) and along the activation
+    rows, a fused activation; then Q8_0H one-hot activations, bit for bit, with -128 planted."""
+    cases = [(10240, n, 2560) for n in (5, 16, 17, 31, 33, 48, 49, 64)]
+    cases += [(6152, 24, 256), (6152, 40, 512), (2001, 9, 1280), (2008, 64, 768), (12288, 20, 4096), (4100, 7, 1024),
+              (2560, 33, 10240)]  # the last has too few rows for this kernel: the tiled one, same answer
+    for i, (M, N, K) in enumerate(cases):
+        rng = np.random.default_rng(3100 + i)
+        w = (rng.standard_normal((M, K)) * 0.05).astype(np.float16)
+        x = rng.standard_normal((1, N, K)).astype(np.float16)
+        for to in (True, False):
+            bias = rng.standard_normal(M if to else N).astype(np.float16) if (i + to) % 3 else None
+            got = gpu_matmul(device, Tensor.from_data(w), Tensor.from_data(x),
+                             None if bias is None else Tensor.from_data(bias), False, True, to)
+            want = oracle.matmul_ref(w, oracle.F16, w.shape, x, oracle.F16, x.shape, bias, False, True, to)
+            check(oracle, got, want, DType.F16, ("f16", M, N, K, to))
+    dt = DType.Q8_0H
+    for i, (M, N, K) in enumerate([(10240, 17, 2560), (10240, 32, 2560), (6152, 24, 256), (2001, 19, 1280),
+                                   (12288, 20, 4096), (8200, 31, 512)]):
+        rng = np.random.default_rng(3200 + i)
+        buf = oracle.make_q8_0h((rng.standard_normal((M, K)) * 0.05).astype(np.float32))
+        x = rng.standard_normal((1, N, K)).astype(np.float16)
+        for to in (True, False):
+            bias = rng.standard_normal(M if to else N).astype(np.float16) if (i + to) % 3 else None
+            got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (M, K)), Tensor.from_data(x),
+                             None if bias is None else Tensor.from_data(bias), False, True, to)
+            want = oracle.matmul_ref(buf, oracle.Q8_0H, (M, K), x, oracle.F16, x.shape, bias, False, True, to)
+            check(oracle, got, want, DType.F16, ("q8_0h", M, N, K, to))
+    # GELU / SiLU behind the Linear, fused
+    rng = np.random.default_rng(3280)
+    M, K, N = 6152, 1024, 24
+    w = (rng.standard_normal((M, K)) * 0.05).astype(np.float16)
+    buf = oracle.make_q8_0h(w.astype(np.float32))
+    x = rng.standard_normal((1, N, K)).astype(np.float16)
+    bias = rng.standard_normal(M).astype(np.float16)
+    for name, act in (("gelu", oracle.ACT_GELU), ("silu", oracle.ACT_SILU)):
+        for wt, odt, src in ((Tensor.from_data(w), oracle.F16, w), (Tensor.from_quantized(buf, dt, (M, K)), oracle.Q8_0H, buf)):
+            y = getattr(wt.to(device).gemm(Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device),
+                                           False, True, True), name)().resolve()
+            want = oracle.matmul_ref(src, odt, (M, K), x, oracle.F16, x.shape, bias, False, True, True, act=act)
+            assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want)), (name, odt)
+    # one-hot: the dequantized weight, bit for bit
+    for M, K in ((10240, 2560), (6152, 256), (2001, 1280)):
+        buf = q8_weight(oracle, rng, M, K, dt)
+        buf[: M * K][5::97] = 0x80
+        dq = oracle.q8_0_dequantize(buf, M * K, True).reshape(M, K)
+        for N in (17, 32):
+            cols = np.concatenate([[5 + 97 * 2], rng.integers(0, K, size=N)])[:N]
+            x = np.zeros((N, K), dtype=np.float16)
+            x[np.arange(N), cols] = 1
+            got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (M, K)), Tensor.from_data(x), None, False, True, True)
+            assert np.array_equal(got, dq[:, cols].T.astype(np.float16)), (M, K, N)
+
+
 def test_f16_nt_gemm_stack_broadcast(device, oracle):
     rng = np.random.default_rng(650)
     a = rng.standard_normal((1, 200, 128)).astype(np.float16)      # one weight, four activation stacks
