@@ -29,6 +29,10 @@
 // dword pair regroups them so that the first MFMA sees only block 2s and the
 // second only block 2s+1; within a block the order of K is irrelevant as long
 // as the activation fragment uses the same order, which x_koff() provides.
+// The regular-case variant loads the same 16 rows x 64 bytes in address order instead (lane l: row l / 4, piece
+// l % 4, so that a quad of lanes reads 64 consecutive bytes and the L1 handles one access per quad, not four) and
+// brings a step to the layout above through a 1 KB LDS slot, the wavefront's slab of the final sums' region
+// (swizzled ds_write_b128, ds_read_b128): 10240 x 2560 at 8 vectors 9.6 -> 9.0 us.
 #include "device_common.h"
 
 namespace rt {
@@ -47,6 +51,7 @@ struct GemvMfmaArgs {
     int64_t b_bs, b_js;
     int64_t o_bs, o_is, o_js;
     int has_bias, bias_on_rows, act;
+    int lin;               // the regular case loads its weights in address order
 };
 
 // K offset (within a 64-wide step) of the 8 values lane group g feeds to the
@@ -72,6 +77,8 @@ __device__ __forceinline__ half8_t cvt_i8x8_f16x8(uint32_t v0, uint32_t v1) {
     return half8_t{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
+RT_TUNABLE(g_gemv_mfma_lin, 1); // 0: the regular case loads its weights in operand order (for comparisons)
+
 constexpr int kUnitK = 256; // K covered by one unit: 4 steps of 64, 8 scale blocks
 constexpr int kXPad = 8;    // halfs of padding per staged row (keeps 16-lane LDS reads conflict-free)
 
@@ -87,8 +94,7 @@ constexpr int kXPad = 8;    // halfs of padding per staged row (keeps 16-lane LD
 // NCT is the compile-time ceiling of the number of activation vectors (it sizes the
 // staging registers).
 // FAST is the regular case, which the launcher recognises: one stack, every one of the
-// workgroup's rows and every one of its wavefronts' units exists, exactly NCT vectors, and all
-// offsets below 2^31.  Its prologue is a handful of 32-bit operations (no clamps, no stack
+// workgroup's rows and every one of its wavefronts' units exists, and all offsets below 2^31.  Its prologue is a handful of 32-bit operations (no clamps, no stack
 // arithmetic), which matters because every wavefront runs it before its first load is issued
 // and several wavefronts per SIMD run it at the same time.
 template <int UPW, int RG, int NCT, bool FAST>
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
     constexpr int XROW = UPW * kUnitK + kXPad; // halfs per staged activation row (this wave's K slice)
     const int t = threadIdx.x, lane = t & 63, nwaves = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6); // wave-uniform: addresses below stay scalar
-    const int NC = FAST ? NCT : g.NC;
+    const int NC = g.NC;
     half_t *xs = (half_t *)smem + (size_t)wave * NC * XROW;          // [NC][XROW], private to this wave
     float *psum = (float *)((half_t *)smem + (size_t)nwaves * NC * XROW); // [nwaves][RG][256]
 
@@ -125,13 +131,15 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
 #pragma unroll
         for (int i = 0; i < XL; i++) {
             const uint32_t v = min(i * 64 + lane, NCT * VPR - 1); // lanes past the end re-read the last vector
-            const uint32_t j = v / VPR, kv = v % VPR;
+            const uint32_t j = min(v / VPR, (uint32_t)NC - 1u), kv = v % VPR; // fewer than NCT vectors: the last one again, never staged
             xv[i] = *(const uint4_t *)(xg + (j * (uint32_t)g.b_js + 8u * kv));
         }
         asm volatile("" ::: "memory"); // keep the loads in this order
         // 2. the weight stream: a wave-uniform 64-bit base plus a 32-bit lane offset
         const uint8_t *qbase = g.qs + ((uint32_t)row0 * (uint32_t)g.K + (uint32_t)(u0 * kUnitK));
-        const uint32_t loff = (uint32_t)n * (uint32_t)g.K + 16u * grp;
+        // address order (RT_MFMA_LIN): a quad of lanes reads 64 consecutive bytes of row lane / 4; the step passes
+        // through an LDS slot on its way to operand order.  Operand order: row lane % 16, piece lane / 16.
+        const uint32_t loff = g.lin ? (uint32_t)(lane >> 2) * (uint32_t)g.K + 16u * (lane & 3) : (uint32_t)n * (uint32_t)g.K + 16u * grp;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
@@ -149,7 +157,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
             for (int u = 0; u < UPW; u++) dsc[rg][u] = *(const uint4_t *)(sbase + ((uint32_t)(16 * rg + n) * kq + u * 8));
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
-            const uint32_t bi = g.bias_on_rows ? (uint32_t)row0 + 16 * rg + (t & 15) : (uint32_t)min((t >> 4) & 15, NCT - 1);
+            const uint32_t bi = g.bias_on_rows ? (uint32_t)row0 + 16 * rg + (t & 15) : (uint32_t)min((t >> 4) & 15, NC - 1);
             const half_t *bp = g.has_bias ? g.bias + bi : sbase;
             bias_raw[rg] = *(const uint16_t *)bp;
         }
@@ -230,9 +238,18 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
                 const half8_t dh = __builtin_bit_cast(half8_t, dsc[rg][u]);
 #pragma unroll
                 for (int st = 0; st < 4; st++) {
+                    uint4_t wq = w[rg][u][st];
+                    if (FAST && g.lin) {
+                        // load order -> operand order through this wavefront's slab of the sums' region (unused until
+                        // the MFMAs are done; one wavefront's DS operations complete in order)
+                        uint8_t *slot = (uint8_t *)(psum + (wave * RG + rg) * 256);
+                        const int lr = lane >> 2, lc = lane & 3;
+                        *(uint4_t *)(slot + lr * 64 + 16 * (lc ^ ((lr >> 2) & 3))) = wq;
+                        wq = *(const uint4_t *)(slot + n * 64 + 16 * (grp ^ ((n >> 2) & 3)));
+                    }
                     // regroup: afterwards p?[0] is this lane's share of block 2*st and p?[1] of block 2*st+1
-                    auto p0 = __builtin_amdgcn_permlane32_swap(w[rg][u][st][0], w[rg][u][st][2], false, false);
-                    auto p1 = __builtin_amdgcn_permlane32_swap(w[rg][u][st][1], w[rg][u][st][3], false, false);
+                    auto p0 = __builtin_amdgcn_permlane32_swap(wq[0], wq[2], false, false);
+                    auto p1 = __builtin_amdgcn_permlane32_swap(wq[1], wq[3], false, false);
                     const half8_t b0 = cvt_i8x8_f16x8(p0[0], p1[0]);
                     const half8_t b1 = cvt_i8x8_f16x8(p0[1], p1[1]);
                     const half8_t a0 = __builtin_bit_cast(half8_t, *(const uint4_t *)(xrow + u * kUnitK + st * 64));
@@ -264,7 +281,7 @@ __global__ __launch_bounds__(1024) void gemv_q8h_mfma_kernel(GemvMfmaArgs g) {
             float v = 0.f;
             for (int w2 = 0; w2 < nwaves; w2++) v += psum[(w2 * RG + rg) * 256 + t];
             const int64_t i = row0 + 16 * rg + (t & 15);
-            if (FAST || (j < g.NC && i < g.M && 16 * rg + (t & 15) < g.rows_wg)) g.out[s * g.o_bs + i * g.o_is + j * g.o_js] = (half_t)rt_act(v + (g.has_bias ? (float)__builtin_bit_cast(half2_t, bias_raw[rg])[0] : 0.f), g.act);
+            if (FAST ? j < g.NC : (j < g.NC && i < g.M && 16 * rg + (t & 15) < g.rows_wg)) g.out[s * g.o_bs + i * g.o_is + j * g.o_js] = (half_t)rt_act(v + (g.has_bias ? (float)__builtin_bit_cast(half2_t, bias_raw[rg])[0] : 0.f), g.act);
         }
     }
 }
@@ -289,7 +306,7 @@ static hipError_t launch_kernel(dim3 grid, int nwaves, size_t lds, hipStream_t s
 template <int UPW, int RG, int NCT>
 static hipError_t launch_one(dim3 grid, int nwaves, size_t lds, hipStream_t st, const GemvMfmaArgs &g) {
     if constexpr (RG == 1) {
-        const bool regular = grid.y == 1 && g.a_stack == 1 && g.b_stack == 1 && g.M % 16 == 0 && g.NC == NCT &&
+        const bool regular = grid.y == 1 && g.a_stack == 1 && g.b_stack == 1 && g.M % 16 == 0 &&
                              g.nunits == nwaves * UPW && g.M * g.K < (int64_t(1) << 31) &&
                              (int64_t)g.NC * g.b_js < (int64_t(1) << 30);
         if (regular) return launch_kernel<UPW, RG, NCT, true>(grid, nwaves, lds, st, g);
@@ -341,7 +358,7 @@ hipError_t launch_gemv_q8h_mfma(const Problem &p, const void *A, const void *B, 
     g.a_stack = p.a_stack, g.b_stack = p.b_stack;
     g.b_bs = p.b_bs, g.b_js = bjs;
     g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
-    g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
+    g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act, g.lin = g_gemv_mfma_lin;
 
     // Units per wavefront: as few as keeps the workgroup within 16 wavefronts.
     int upw = g_gemv_mfma_upw;

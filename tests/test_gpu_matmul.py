@@ -201,6 +201,41 @@ def test_q8_streaming_regular_and_ragged_variants(device, oracle):
     assert np.array_equal(got, dq[:, cols].T.astype(adt))
 
 
+def test_q8_streaming_regular_variant_below_its_vector_ceiling(device, oracle):
+    """5, 6, 7 (ceiling 8) and 3 (ceiling 4, K too long for the 4x4x4 kernel) vectors against whole 16-row groups run
+    the regular variant, which loads the weights in address order and turns them to operand order through LDS: the
+    bias along the rows and along the vectors (read at indices below the vector count only), GELU fused, and
+    one-hot activations bit for bit with -128 planted."""
+    dt = DType.Q8_0H
+    for i, (M, N, K) in enumerate([(5, 10240, 2560), (6, 4096, 2560), (7, 640, 5120), (3, 2048, 8192), (8, 10240, 2560)]):
+        rng = np.random.default_rng(2700 + i)
+        buf = q8_weight(oracle, rng, N, K, dt)
+        x = rng.standard_normal((1, M, K)).astype(np.float16)
+        for to in (True, False):
+            bias = rng.standard_normal(N if to else M).astype(np.float16)
+            got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (N, K)), Tensor.from_data(x), Tensor.from_data(bias),
+                             False, True, to)
+            want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, bias, False, True, to)
+            check(oracle, got, want, DType.F16, (M, N, K, to))
+    N, K = 4096, 2560
+    rng = np.random.default_rng(2750)
+    buf = q8_weight(oracle, rng, N, K, dt)
+    x = rng.standard_normal((1, 6, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    y = Tensor.from_quantized(buf, dt, (N, K)).to(device).gemm(Tensor.from_data(x).to(device), Tensor.from_data(bias).to(device),
+                                                                False, True, True).gelu().resolve()
+    want = oracle.matmul_ref(buf, oracle.Q8_0H, (N, K), x, oracle.F16, x.shape, bias, False, True, True, act=oracle.ACT_GELU)
+    assert np.all(np.abs(y.to(Device.CPU).storage.astype(np.float64) - want) <= 2e-3 + 2e-2 * np.abs(want))
+    buf[: N * K][5::97] = 0x80
+    dq = oracle.q8_0_dequantize(buf, N * K, True).reshape(N, K)
+    for M in (5, 7, 8):
+        cols = np.concatenate([[5 + 97 * 3], rng.integers(0, K, size=M)])[:M]
+        x = np.zeros((M, K), dtype=np.float16)
+        x[np.arange(M), cols] = 1
+        got = gpu_matmul(device, Tensor.from_quantized(buf, dt, (N, K)), Tensor.from_data(x), None, False, True, True)
+        assert np.array_equal(got, dq[:, cols].T.astype(np.float16)), M
+
+
 def test_q8_streaming_rows_dealt_one_workgroup_per_compute_unit(device, oracle):
     """With 9..16 vectors the activations' LDS lets one or two workgroups of the Q8_0H streaming kernel live on a
     compute unit; when the 16-row workgroups would then run in rounds, every compute unit gets one workgroup with
