@@ -618,17 +618,19 @@ def other_configs(r: Runner, O):
     out.append(bench_decoder_layer(r, O))
     out.append(bench_decoder_layer(r, O, fused_qkv=True))
     out += bench_q4k(r, O, (1, 16, 128, 256), 200)
-    # a short prompt against the C4 up-projection: 128 activation rows run on 64-row weight tiles so that every
-    # compute unit has a workgroup (160 workgroups; the 160-row tile would leave 64)
+    # short prompts against the C4 up-projection, the weights from HBM: 16 / 32 / 64 rows on the weight-streaming
+    # GEMM (Q8_0H at 16 rows on the streaming GEMV, at 64 on 64-row tiles), 128 rows on 64-row weight tiles so that
+    # every compute unit has a workgroup (160 workgroups; the 160-row tile would leave 64)
     rng = np.random.default_rng(8)
     w = (rng.standard_normal((10240, 2560)) * 0.02).astype(np.float32)
-    x = rng.standard_normal((1, 128, 2560)).astype(np.float16)
     bias = rng.standard_normal(10240).astype(np.float16)
-    for name, lhs, dt, wbytes in (("f16", w.astype(np.float16), ffi.RT_F16, 10240 * 2560 * 2),
-                                  ("Q8_0H", O.make_q8_0h(w), ffi.RT_Q8_0H, 10240 * 2560 * 17 // 16)):
-        out.append(bench_generic(r, O, f"C4 up at 128 rows: X[128x2560] f16 . {name} W[10240x2560]^T + bias", lhs, dt,
-                                 (10240, 2560), x, x.shape, bias, (False, True, True), np.float16, 2.0 * 128 * 10240 * 2560,
-                                 wbytes + (128 * 2560 + 10240 + 128 * 10240) * 2, 100, 2e-2))
+    for rows in (16, 32, 64, 128):
+        x = rng.standard_normal((1, rows, 2560)).astype(np.float16)
+        for name, lhs, dt, wbytes in (("f16", w.astype(np.float16), ffi.RT_F16, 10240 * 2560 * 2),
+                                      ("Q8_0H", O.make_q8_0h(w), ffi.RT_Q8_0H, 10240 * 2560 * 17 // 16)):
+            out.append(bench_generic(r, O, f"C4 up at {rows} rows: X[{rows}x2560] f16 . {name} W[10240x2560]^T + bias", lhs, dt,
+                                     (10240, 2560), x, x.shape, bias, (False, True, True), np.float16, 2.0 * rows * 10240 * 2560,
+                                     wbytes + (rows * 2560 + 10240 + rows * 10240) * 2, 100, 2e-2))
     return out
 
 
