@@ -775,14 +775,16 @@ def test_f16_weights_few_activation_rows(device, oracle):
 
 
 def test_weight_streaming_short_prompts(device, oracle):
-    """f16 weights against 5..64 and Q8_0H weights against 17..32 activation rows, K a multiple of 256 and enough
+    """f16 weights against 5..96 and Q8_0H weights against 17..48 activation rows, K a multiple of 256 and enough
     weight rows for three quarters of the compute units, take the weight-streaming GEMM: every tile count of
     activation rows (and counts off the 16 of a tile), one to three tiles of weight rows per workgroup, row counts
     off the 8 of a share (the scalar output path) and off the 16 of a tile, K from one step per wavefront (256) to
-    more steps than the register ring holds, the bias along the weight rows (trans_out) and along the activation
-    rows, a fused activation; then Q8_0H one-hot activations, bit for bit, with -128 planted."""
-    cases = [(10240, n, 2560) for n in (5, 16, 17, 31, 33, 48, 49, 64)]
+    more steps than the weight loader's register ring holds (and step counts off its four), the bias along the
+    weight rows (trans_out) and along the activation rows, a fused activation; then Q8_0H one-hot activations, bit
+    for bit, with -128 planted."""
+    cases = [(10240, n, 2560) for n in (5, 16, 17, 31, 33, 48, 49, 64, 65, 80, 96, 97)]
     cases += [(6152, 24, 256), (6152, 40, 512), (2001, 9, 1280), (2008, 64, 768), (12288, 20, 4096), (4100, 7, 1024),
+              (6152, 90, 1536), (8200, 70, 3328),
               (2560, 33, 10240)]  # the last has too few rows for this kernel: the tiled one, same answer
     for i, (M, N, K) in enumerate(cases):
         rng = np.random.default_rng(3100 + i)
@@ -796,7 +798,8 @@ def test_weight_streaming_short_prompts(device, oracle):
             check(oracle, got, want, DType.F16, ("f16", M, N, K, to))
     dt = DType.Q8_0H
     for i, (M, N, K) in enumerate([(10240, 17, 2560), (10240, 32, 2560), (6152, 24, 256), (2001, 19, 1280),
-                                   (12288, 20, 4096), (8200, 31, 512)]):
+                                   (12288, 20, 4096), (8200, 31, 512), (10240, 33, 2560), (10240, 48, 2560),
+                                   (10240, 49, 2560), (6152, 40, 1536)]):
         rng = np.random.default_rng(3200 + i)
         buf = oracle.make_q8_0h((rng.standard_normal((M, K)) * 0.05).astype(np.float32))
         x = rng.standard_normal((1, N, K)).astype(np.float16)
@@ -824,7 +827,7 @@ def test_weight_streaming_short_prompts(device, oracle):
         buf = q8_weight(oracle, rng, M, K, dt)
         buf[: M * K][5::97] = 0x80
         dq = oracle.q8_0_dequantize(buf, M * K, True).reshape(M, K)
-        for N in (17, 32):
+        for N in (17, 32, 48):
             cols = np.concatenate([[5 + 97 * 2], rng.integers(0, K, size=N)])[:N]
             x = np.zeros((N, K), dtype=np.float16)
             x[np.arange(N), cols] = 1
