@@ -16,7 +16,8 @@
 //     stages, swizzled the same way on the global side.
 // One workgroup barrier per step.  Before barrier h the activation loader has seen stage (h + 1) % SX land, the
 // weight loader has written slot (h + 1) % 2, the multiplying wavefront has read slot h % 2 and stage h % SX for
-// the last time.
+// the last time.  From five tiles of activation rows (f16 weights) K is split in halves instead and the two
+// multiplying wavefronts of a half take half of the activation tiles each: see the kernel's NK.
 //
 // Why three roles.  A wavefront issues in order: one that cannot issue its next load (the compute unit's vector
 // memory pipeline pushes back when its queue is full) cannot issue its MFMAs either.  With every wavefront loading
@@ -74,31 +75,32 @@ constexpr int gs_vmcnt(int n) { return 0x0F70 | (n & 0xF) | (((n >> 4) & 0x3) <<
 // The K ranges meet.  Called by the four multiplying wavefronts (threads 0..255) once nothing of theirs is on its way
 // into LDS; three workgroup barriers (two when the output is not vectorised), which any other wavefront of the
 // workgroup must match with gs_epilogue_barriers().
-template <int TA, int TB>
-__device__ __forceinline__ void gs_epilogue(const GemmStreamArgs &g, float4_t (&acc)[TA][TB], uint8_t *smem, int wave, int lane, int t,
-                                            int64_t row0, int last, const uint16_t (&bias_raw)[TA]) {
+template <int TA, int TB, int NK>
+__device__ __forceinline__ void gs_epilogue(const GemmStreamArgs &g, float4_t (&acc)[TA][TB / (4 / NK)], uint8_t *smem, int kpart, int bgrp,
+                                            int lane, int t, int64_t row0, int last, const uint16_t (&bias_raw)[TA]) {
+    constexpr int TBW = TB / (4 / NK); // activation tiles of one multiplying wavefront
     const int fr = lane & 15, fg = lane >> 4;
     __syncthreads(); // every wavefront is done with its ring: the regions change hands
-    // every wavefront leaves its sums, then takes every fourth tile
-    float4_t *red = (float4_t *)smem;                             // [wave][TA * TB][64]
-    half_t *Os = (half_t *)(smem + (size_t)4 * TA * TB * 1024);   // [16 TB][16 TA + 8]
+    // every wavefront leaves its sums; the NK wavefronts that hold parts of the same tiles then take every NK-th of them
+    float4_t *red = (float4_t *)smem;                             // [K part][TA * TB][64]
+    half_t *Os = (half_t *)(smem + (size_t)NK * TA * TB * 1024);  // [16 TB][16 TA + 8]
     constexpr int OLD = 16 * TA + 8;
 #pragma unroll
     for (int a = 0; a < TA; a++)
 #pragma unroll
-        for (int b = 0; b < TB; b++) red[(wave * TA * TB + a * TB + b) * 64 + lane] = acc[a][b];
+        for (int b = 0; b < TBW; b++) red[(kpart * TA * TB + a * TB + bgrp * TBW + b) * 64 + lane] = acc[a][b];
     __syncthreads();
     half_t *out = g.out;
     const bool vec_out = g.vec_out != 0;
     rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
-        for (int idx = 0; idx < TA * TB; idx++) {
-            if ((idx & 3) != wave) continue; // wave-uniform
-            const int a = idx / TB, b = idx % TB;
-            float4_t v = red[idx * 64 + lane];
+        for (int idx = 0; idx < TA * TBW; idx++) {
+            if ((idx & (NK - 1)) != kpart) continue; // wave-uniform
+            const int a = idx / TBW, b = bgrp * TBW + idx % TBW;
+            float4_t v = red[(a * TB + b) * 64 + lane];
 #pragma unroll
-            for (int w2 = 1; w2 < 4; w2++) {
-                const float4_t o = red[(w2 * TA * TB + idx) * 64 + lane];
+            for (int w2 = 1; w2 < NK; w2++) {
+                const float4_t o = red[(w2 * TA * TB + a * TB + b) * 64 + lane];
 #pragma unroll
                 for (int r = 0; r < 4; r++) v[r] += o[r];
             }
@@ -138,26 +140,33 @@ __device__ __forceinline__ void gs_epilogue_barriers(const GemmStreamArgs &g) {
 // rows' two block scales, a dword per row)
 template <int TA, bool Q8> constexpr int gs3_wslot() { return Q8 ? TA * 16 * 64 + 256 : TA * 16 * 128; }
 template <int TA, int TB, int SX, bool Q8> constexpr int gs3_pair_lds() { return SX * 16 * TB * 128 + 2 * gs3_wslot<TA, Q8>(); }
-template <int TA, int TB, int SX, bool Q8> constexpr size_t gs3_lds_bytes() {
-    constexpr size_t ring = (size_t)4 * gs3_pair_lds<TA, TB, SX, Q8>();
-    constexpr size_t red = (size_t)4 * TA * TB * 1024 + (size_t)16 * TB * (16 * TA + 8) * 2;
+template <int TA, int TB, int SX, bool Q8, int NK> constexpr size_t gs3_lds_bytes() {
+    constexpr size_t ring = (size_t)NK * gs3_pair_lds<TA, TB, SX, Q8>();
+    constexpr size_t red = (size_t)NK * TA * TB * 1024 + (size_t)16 * TB * (16 * TA + 8) * 2;
     return ring > red ? ring : red;
 }
 
-// TA / TB: tiles of 16 weight rows / activation rows; SX: activation stages; DW: steps the weight loads run ahead; Q8: Q8_0H weights
-template <int TA, int TB, int SX, int DW, bool Q8>
+// TA / TB: tiles of 16 weight rows / activation rows; SX: activation stages; DW: steps the weight loads run ahead; Q8: Q8_0H weights.
+// NK: parts of K (4 or 2).  With K in halves the two multiplying wavefronts of a half take half of the activation tiles
+// each (both read every weight fragment), each half has two weight and two activation loaders that deal its load
+// instructions between them, there are half as many rings to hold and half as many partial sums to add: the form for
+// six and eight tiles of activation rows, whose stages are too large for four rings.
+template <int TA, int TB, int SX, int DW, bool Q8, int NK>
 __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
+    static_assert(NK == 4 || (NK == 2 && !Q8 && TB % 2 == 0), "K in quarters, or in halves for f16 weights and an even tile count");
+    constexpr int NB = 4 / NK, TBW = TB / NB, NLS = 4 / NK; // wavefronts per K part: multiplying, and loading of either kind
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int t = threadIdx.x, lane = t & 63;
     const int wv = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int role = wv >> 2, wave = wv & 3; // 0 multiplies, 1 loads weights, 2 loads activations; `wave`: the K quarter
+    const int role = wv >> 2; // 0 multiplies, 1 loads weights, 2 loads activations
+    const int wave = (wv & 3) / NB, sub = (wv & 3) % NB; // the K part; the wavefront's number among its kind in that part
     const int fr = lane & 15, fg = lane >> 4;
     const int64_t row0 = (int64_t)blockIdx.x * g.rows_wg;
     const int last = (int)min((int64_t)g.rows_wg, g.M - row0) - 1; // rows past the share's end repeat its last row; never stored
-    const uint32_t K = (uint32_t)g.K, kq = K >> 2;
+    const uint32_t K = (uint32_t)g.K, kq = K / NK;
     const int nh = (int)(kq >> 6); // steps of 64 values of K
     constexpr int XSTAGE = 16 * TB * 128, WSLOT = gs3_wslot<TA, Q8>();
-    constexpr int XLD = 2 * TB, WLD = Q8 ? TA : 2 * TA;
+    constexpr int XLD = 2 * TB / NLS, WLD = (Q8 ? TA : 2 * TA) / NLS; // load instructions per step and loading wavefront
     uint8_t *xring = smem + wave * gs3_pair_lds<TA, TB, SX, Q8>();
     uint8_t *wslots = xring + SX * XSTAGE;
 
@@ -166,7 +175,7 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
         uint32_t xsrc[XLD];
 #pragma unroll
         for (int i = 0; i < XLD; i++) {
-            const int row = 8 * i + (lane >> 3);
+            const int row = 8 * (i * NLS + sub) + (lane >> 3);
             const int c = (lane & 7) ^ ((row >> 1) & 7);
             xsrc[i] = ((uint32_t)min((int64_t)row, g.N - 1) * (uint32_t)g.b_js + 8u * c) * 2u;
         }
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
 #pragma unroll
             for (int i = 0; i < XLD; i++)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xs + xsrc[i]),
-                                                 (__attribute__((address_space(3))) void *)(xring + stage * XSTAGE + i * 1024), 16, 0, 0);
+                                                 (__attribute__((address_space(3))) void *)(xring + stage * XSTAGE + (i * NLS + sub) * 1024), 16, 0, 0);
         };
         const int lasth = nh - 1;
 #pragma unroll
@@ -208,7 +217,7 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
         uint32_t woff[WLD], wst[WLD];
 #pragma unroll
         for (int i = 0; i < WLD; i++) {
-            const int rl = Q8 ? 16 * i + (lane >> 2) : 8 * i + (lane >> 3), c = Q8 ? lane & 3 : lane & 7;
+            const int rl = Q8 ? 16 * (i * NLS + sub) + (lane >> 2) : 8 * (i * NLS + sub) + (lane >> 3), c = Q8 ? lane & 3 : lane & 7;
             woff[i] = Q8 ? (uint32_t)min(rl, last) * K + 16u * c : (uint32_t)min(rl, last) * K * 2u + 16u * c;
             wst[i] = Q8 ? (uint32_t)(rl * 64 + 16 * (c ^ ((rl >> 2) & 3))) : (uint32_t)(rl * 128 + 16 * (c ^ ((rl >> 1) & 7)));
         }
@@ -272,12 +281,12 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
         const uint16_t *bp = (g.has_bias && g.bias_on_rows) ? (const uint16_t *)g.bias + min(row0 + 16 * a + fr, g.M - 1) : (const uint16_t *)g.W;
         bias_raw[a] = *bp;
     }
-    float4_t acc[TA][TB];
+    float4_t acc[TA][TBW];
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int a = 0; a < TA; a++)
 #pragma unroll
-        for (int b = 0; b < TB; b++) acc[a][b] = zero;
+        for (int b = 0; b < TBW; b++) acc[a][b] = zero;
     // operand-order reads: lane (fr, fg) wants pieces pc and 4 + pc of row 16 tile + fr (Q8_0H: lane group fg feeds the
     // first MFMA of a step with K offsets 16 (fg & 1) + 8 (fg >> 1), the second with + 32; its 16 codes are piece fg)
     const int pc = Q8 ? 2 * (fg & 1) + (fg >> 1) : fg;
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
     int stage = 0;
     for (int h = 0; h < nh; h++) {
         asm volatile("" ::: "memory");
-        const uint8_t *ws = wslots + (h & 1) * WSLOT, *xs = xring + stage * XSTAGE;
+        const uint8_t *ws = wslots + (h & 1) * WSLOT, *xs = xring + stage * XSTAGE + sub * (TBW * 2048);
         half8_t wf[TA][2];
         float d0[Q8 ? TA : 1], d1[Q8 ? TA : 1];
         if constexpr (Q8) {
@@ -312,8 +321,8 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
         xf[0][0] = __builtin_bit_cast(half8_t, *(const uint4_t *)(xs + rd0));
         xf[0][1] = __builtin_bit_cast(half8_t, *(const uint4_t *)(xs + rd1));
 #pragma unroll
-        for (int b = 0; b < TB; b++) {
-            if (b + 1 < TB) {
+        for (int b = 0; b < TBW; b++) {
+            if (b + 1 < TBW) {
                 xf[(b + 1) & 1][0] = __builtin_bit_cast(half8_t, *(const uint4_t *)(xs + (b + 1) * 2048 + rd0));
                 xf[(b + 1) & 1][1] = __builtin_bit_cast(half8_t, *(const uint4_t *)(xs + (b + 1) * 2048 + rd1));
             }
@@ -337,50 +346,59 @@ __global__ __launch_bounds__(768) void gemm_stream_kernel(GemmStreamArgs g) {
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this step's fragment reads have returned
         __builtin_amdgcn_s_barrier();       // barrier h
     }
-    gs_epilogue<TA, TB>(g, acc, smem, wave, lane, t, row0, last, bias_raw);
+    gs_epilogue<TA, TB, NK>(g, acc, smem, wave, sub, lane, t, row0, last, bias_raw);
 }
 
 RT_TUNABLE(g_gemm_stream_disable, 0); // non-zero keeps short prompts on the tiled kernels (for comparisons)
 RT_TUNABLE(g_gemm_stream_max_n, 0);   // activation rows up to which the kernel takes a product (0: the measured crossovers)
 
-template <int TA, int TB, bool Q8> static hipError_t gs_launch(const GemmStreamArgs &g, unsigned nwg, hipStream_t stream) {
-    // as many activation stages as fit 40 KB per K quarter beside the two weight slots, at most 6.  The weight loads
-    // run four steps ahead (2 or 6: the same to 2 %).
-    constexpr int SXfit = (40 * 1024 - 2 * gs3_wslot<TA, Q8>()) / (16 * TB * 128), SX = SXfit > 6 ? 6 : SXfit;
+template <int TA, int TB, bool Q8, int NK> static hipError_t gs_launch(const GemmStreamArgs &g, unsigned nwg, hipStream_t stream) {
+    // as many activation stages as fit a K part's share of 160 KB beside its two weight slots, at most 6.  The weight
+    // loads run four steps ahead (2 or 6: the same to 2 %).
+    constexpr int SXfit = (160 * 1024 / NK - 2 * gs3_wslot<TA, Q8>()) / (16 * TB * 128), SX = SXfit > 6 ? 6 : SXfit;
     static_assert(SX >= 2, "a stage to fill while one is read");
-    constexpr size_t lds = gs3_lds_bytes<TA, TB, SX, Q8>();
+    constexpr size_t lds = gs3_lds_bytes<TA, TB, SX, Q8, NK>();
     static_assert(lds <= 160 * 1024, "one workgroup's rings fit a compute unit's LDS");
     if (lds > 48 * 1024) {
-        if (const hipError_t e = ensure_lds_limit<&gemm_stream_kernel<TA, TB, SX, 4, Q8>>(); e != hipSuccess) return e;
+        if (const hipError_t e = ensure_lds_limit<&gemm_stream_kernel<TA, TB, SX, 4, Q8, NK>>(); e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((gemm_stream_kernel<TA, TB, SX, 4, Q8>), dim3(nwg), dim3(768), lds, stream, g);
+    hipLaunchKernelGGL((gemm_stream_kernel<TA, TB, SX, 4, Q8, NK>), dim3(nwg), dim3(768), lds, stream, g);
     return hipGetLastError();
 }
 
+RT_TUNABLE(g_gemm_stream_halves_from, 5); // activation tiles from which f16 weights take K in halves
+
 template <int TA, bool Q8> static hipError_t gs_tb(int tb, const GemmStreamArgs &g, unsigned nwg, hipStream_t stream) {
+    if constexpr (!Q8) {
+        // f16 weights, five to eight tiles of activation rows: K in halves (10240 x 2560: 80 / 96 rows 19.8 / 20.4 us against
+        // 21.2 / 21.4 with K in quarters, 64 rows 18.0 against 17.2; 112 / 128 rows, which do not fit four rings, 22.0 / 22.2)
+        if (tb >= g_gemm_stream_halves_from) {
+            if (tb <= 6) return gs_launch<TA, 6, Q8, 2>(g, nwg, stream);
+            if (tb <= 8) return gs_launch<TA, 8, Q8, 2>(g, nwg, stream);
+        }
+    }
     switch (tb) {
-    case 1: return gs_launch<TA, 1, Q8>(g, nwg, stream);
-    case 2: return gs_launch<TA, 2, Q8>(g, nwg, stream);
-    case 3: return gs_launch<TA, 3, Q8>(g, nwg, stream);
-    case 4: return gs_launch<TA, 4, Q8>(g, nwg, stream);
+    case 1: return gs_launch<TA, 1, Q8, 4>(g, nwg, stream);
+    case 2: return gs_launch<TA, 2, Q8, 4>(g, nwg, stream);
+    case 3: return gs_launch<TA, 3, Q8, 4>(g, nwg, stream);
+    case 4: return gs_launch<TA, 4, Q8, 4>(g, nwg, stream);
     case 5:
-    case 6: return gs_launch<TA, 6, Q8>(g, nwg, stream);
+    case 6: return gs_launch<TA, 6, Q8, 4>(g, nwg, stream);
     }
     return hipErrorNotSupported;
 }
 
 // f16 or Q8_0H weights (rows of K), K-contiguous f16 activations, one stack.
 // Measured at 10240 x 2560 with the weights from HBM (this kernel / the tiled one, us): f16 weights 16 rows 12.5 / 16.1,
-// 32: 14.4 / 17.7, 48: 16.1 / 19.3, 64: 17.3 / 20.5, 96: 21.3 / 25.2, 128 (with one weight slot and two barriers per
-// step, since its two activation stages leave no room for a second slot): 26.8 / 27.3, not kept; Q8_0H 16: 11.9 /
+// 32: 14.4 / 17.7, 48: 16.1 / 19.3, 64: 17.3 / 20.5, 96: 20.4 / 25.2, 112: 22.0 / 26.5, 128: 22.2 / 27.2; Q8_0H 16: 11.9 /
 // 15.8 (the streaming GEMV: 10.8), 32: 14.1 / 16.4, 48: 16.5 / 17.0, 64: 17.8 / 17.7, 96: 22.6 / 21.3.
 // hipErrorNotSupported: another kernel must take the problem.
 hipError_t launch_gemm_stream(const Problem &p, const void *A, const void *B, const void *bias, void *out, hipStream_t stream,
                               const DeviceInfo &dev) {
     const bool q8 = p.a_dt == RT_Q8_0H, f16 = p.a_dt == RT_F16;
     if (g_gemm_stream_disable || (!q8 && !f16) || p.act_dt != RT_F16) return hipErrorNotSupported;
-    const int64_t max_n = g_gemm_stream_max_n ? g_gemm_stream_max_n : (q8 ? 48 : 96);
-    if (p.stacks != 1 || p.N < 1 || p.N > max_n || p.N > 96 || p.K % 256 != 0 || p.K < 256 || p.b_ks != 1) return hipErrorNotSupported;
+    const int64_t max_n = g_gemm_stream_max_n ? g_gemm_stream_max_n : (q8 ? 48 : 128);
+    if (p.stacks != 1 || p.N < 1 || p.N > max_n || p.N > (q8 ? 96 : 128) || p.K % 256 != 0 || p.K < 256 || p.b_ks != 1) return hipErrorNotSupported;
     if (f16 && (p.a_ks != 1 || p.a_rs != p.K)) return hipErrorNotSupported;
     if (((uintptr_t)A & 15u) || ((uintptr_t)B & 15u) || (p.b_js * 2) % 16) return hipErrorNotSupported;
     // every compute unit gets one workgroup with its share of the rows, up to 48; more rows: whole rounds of such shares
@@ -391,7 +409,7 @@ hipError_t launch_gemm_stream(const Problem &p, const void *A, const void *B, co
     const int64_t nwg = (p.M + rows_wg - 1) / rows_wg;
     // a weight with so few rows that a quarter of the compute units would stay idle is the tiled kernels' (they cut K)
     if (nwg * 4 < (int64_t)dev.num_cus * 3 || ta > 3) return hipErrorNotSupported;
-    // a share's offsets are 32-bit: 48 rows of K, 96 activation rows of b_js
+    // a share's offsets are 32-bit: 48 rows of K, 128 activation rows of b_js
     if ((int64_t)rows_wg * p.K * 2 >= (int64_t(1) << 31) || p.N * p.b_js * 2 >= (int64_t(1) << 31)) return hipErrorNotSupported;
     GemmStreamArgs g{};
     g.W = (const uint8_t *)A;

@@ -775,16 +775,16 @@ def test_f16_weights_few_activation_rows(device, oracle):
 
 
 def test_weight_streaming_short_prompts(device, oracle):
-    """f16 weights against 5..96 and Q8_0H weights against 17..48 activation rows, K a multiple of 256 and enough
+    """f16 weights against 5..128 and Q8_0H weights against 17..48 activation rows, K a multiple of 256 and enough
     weight rows for three quarters of the compute units, take the weight-streaming GEMM: every tile count of
     activation rows (and counts off the 16 of a tile), one to three tiles of weight rows per workgroup, row counts
     off the 8 of a share (the scalar output path) and off the 16 of a tile, K from one step per wavefront (256) to
     more steps than the weight loader's register ring holds (and step counts off its four), the bias along the
     weight rows (trans_out) and along the activation rows, a fused activation; then Q8_0H one-hot activations, bit
     for bit, with -128 planted."""
-    cases = [(10240, n, 2560) for n in (5, 16, 17, 31, 33, 48, 49, 64, 65, 80, 96, 97)]
+    cases = [(10240, n, 2560) for n in (5, 16, 17, 31, 33, 48, 49, 64, 65, 80, 96, 97, 112, 113, 128, 129)]
     cases += [(6152, 24, 256), (6152, 40, 512), (2001, 9, 1280), (2008, 64, 768), (12288, 20, 4096), (4100, 7, 1024),
-              (6152, 90, 1536), (8200, 70, 3328),
+              (6152, 90, 1536), (8200, 70, 3328), (2008, 128, 256), (4096, 100, 768), (12288, 120, 1280), (2001, 77, 512),
               (2560, 33, 10240)]  # the last has too few rows for this kernel: the tiled one, same answer
     for i, (M, N, K) in enumerate(cases):
         rng = np.random.default_rng(3100 + i)
