@@ -88,18 +88,34 @@ __device__ __forceinline__ float at_groups_sum(float v) {
     return __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
 }
 
-// DP: head_dim padded to a multiple of 32.  MASK: an additive mask tensor is present.
+constexpr int at_stages(int dp) { return dp <= 96 ? 4 : 3; } // stages of the key / value ring
+
+// four transposing reads at two addresses with immediate offsets; nothing waits here
+template <int O0, int O1, int O2, int O3>
+__device__ __forceinline__ void at_tr_read4(uint64_t &v0, uint64_t &v1, uint64_t &v2, uint64_t &v3, uint32_t a0, uint32_t a1) {
+    asm volatile("ds_read_b64_tr_b16 %0, %4 offset:%6\n\tds_read_b64_tr_b16 %1, %4 offset:%7\n\t"
+                 "ds_read_b64_tr_b16 %2, %5 offset:%8\n\tds_read_b64_tr_b16 %3, %5 offset:%9"
+                 : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+                 : "v"(a0), "v"(a1), "n"(O0), "n"(O1), "n"(O2), "n"(O3)
+                 : "memory");
+}
+
+// DP: head_dim padded to a multiple of 32.  MASK: an additive mask tensor is present.  DC: head_dim itself when the
+// kernel is built for one (64, 80, 96, 128), else 0 and head_dim is the argument's: with a constant row length the
+// fragment addresses inside a stage differ by constants, which the LDS instructions carry as immediate offsets, so
+// a block costs three address additions instead of eighteen.
 // Eight wavefronts: wavefront (qt, kh) owns query tile qt (16 rows) and half kh (32 keys) of every
 // key block, with its own running maximum, sum and output; the two halves of a row are merged
 // through LDS at the end.  Two wavefronts per SIMD hide each other's latencies.
-template <int DP, bool MASK>
+template <int DP, bool MASK, int DC>
 __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
+    static_assert(DC == 0 || (DC % 8 == 0 && DC <= DP && DC > DP - 32), "a fixed head_dim belongs to its padded size");
     constexpr int KK = DP / 32;             // MFMA steps over head_dim
     constexpr int DT = DP / 16;             // 16-column tiles of the output
     // load instructions per wavefront per block: a block is 2 * dvec instructions (64 chunks each,
     // keys then values); instruction j belongs to wavefront j % 8, surplus ones repeat the last
     constexpr int NI = (2 * (DP / 8) + AT_WAVES - 1) / AT_WAVES;
-    constexpr int STAGES = DP <= 96 ? 4 : 3;
+    constexpr int STAGES = at_stages(DP);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int t = threadIdx.x, lane = t & 63;
@@ -112,10 +128,11 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     const half_t *K = g.K + b * g.k_bs + h * g.k_hs;
     const half_t *V = g.V + b * g.v_bs + h * g.v_hs;
     half_t *O = g.O + b * g.o_bs + h * g.o_hs;
-    const int dvec = g.D >> 3;              // 16-byte chunks per row (head_dim % 8 == 0)
+    const int D = DC ? DC : g.D;
+    const int dvec = D >> 3;                // 16-byte chunks per row (head_dim % 8 == 0)
     const int off = g.kv_len - g.q_len;     // causal: query i sees keys <= i + off
     const uint4_t zero4 = {0u, 0u, 0u, 0u};
-    const int blk_halfs = AT_BK * g.D;      // one packed block of keys (or values)
+    const int blk_halfs = AT_BK * D;        // one packed block of keys (or values)
     half_t *ring = (half_t *)smem;          // [STAGES][keys | values][64 rows][D]
 
     // this wavefront's Q fragments: row q0 + 16 qt + fr, head_dim 32 kk + 8 fg .. + 7 (zero past head_dim)
@@ -126,7 +143,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
             const int d = 32 * kk + 8 * fg;
-            fq[kk] = d < g.D ? __builtin_bit_cast(half8_t, *(const uint4_t *)(qp + d)) : __builtin_bit_cast(half8_t, zero4);
+            fq[kk] = d < D ? __builtin_bit_cast(half8_t, *(const uint4_t *)(qp + d)) : __builtin_bit_cast(half8_t, zero4);
         }
     }
 
@@ -149,10 +166,23 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
         lcol[i] = 8u * (uint32_t)src;
         ldst[i] = (lval[i] ? blk_halfs : 0) + 512 * jj;
     }
-    // block `src_kb` into the stage of ring position `pos_kb` (they differ only past the end)
+    // block `src_kb` into the stage of ring position `pos_kb` (they differ only past the end).  A block that lies
+    // wholly inside the keys is addressed as a uniform base (the block's first row: scalar arithmetic) plus the
+    // lane's fixed 32-bit byte offset inside a block, so a load costs no vector instruction beside itself.
+    uint32_t lofs[NI];     // byte offset of the lane's chunk from the block's first row
+#pragma unroll
+    for (int i = 0; i < NI; i++) lofs[i] = ((uint32_t)lrow[i] * (uint32_t)(lval[i] ? g.v_rs : g.k_rs) + lcol[i]) * 2u;
     auto issue_loads_at = [&](int pos_kb, int src_kb) {
         half_t *st = ring + (pos_kb % STAGES) * (2 * blk_halfs);
         const int k0 = src_kb * AT_BK;
+        if (k0 + AT_BK <= g.kv_len) { // uniform
+            const uint8_t *kb0 = (const uint8_t *)(K + (int64_t)k0 * g.k_rs), *vb0 = (const uint8_t *)(V + (int64_t)k0 * g.v_rs);
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((lval[i] ? vb0 : kb0) + lofs[i]),
+                                                 (__attribute__((address_space(3))) void *)(st + ldst[i]), 16, 0, 0);
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NI; i++) {
             // rows past the last key re-read the last key: finite data, and their scores are masked
@@ -195,22 +225,22 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     const half_t *mrow = nullptr;
     if constexpr (MASK) mrow = (const half_t *)g.mask; // indexed below by its own element type
     if (nkb > 0) publish(std::integral_constant<int, STAGES - 2>{});
-    // fragment addressing inside a stage (halfs)
-    int koff[2][KK];       // key fragments: row 32 kh + 16 b2 + fr, chunk 4 kk + fg (clamped into the row: Q is zero there)
+    // fragment addressing inside a stage (halfs).  Sixteen rows further down the swizzle repeats, so the second key
+    // tile and the second half of the value rows are 16 dvec chunks away from the first.
+    const int tile_halfs = 128 * dvec;
+    int koff[KK];          // key fragments: row 32 kh + fr (+ 16), chunk 4 kk + fg (clamped into the row: Q is zero there)
 #pragma unroll
-    for (int b2 = 0; b2 < 2; b2++)
+    for (int kk = 0; kk < KK; kk++) koff[kk] = 8 * at_chunk_pos(32 * kh + fr, min(4 * kk + fg, dvec - 1), dvec);
+    int voff[DT];          // value fragments: rows 32 kh + 4 fg + fr / 4 (+ 16), halfs 16 d + 4 (fr % 4) .. + 3
 #pragma unroll
-        for (int kk = 0; kk < KK; kk++)
-            koff[b2][kk] = 8 * at_chunk_pos(32 * kh + 16 * b2 + fr, min(4 * kk + fg, dvec - 1), dvec);
-    int voff[DT][2];       // value fragments: rows 32 kh + 4 fg + fr / 4 (+ 16), halfs 16 d + 4 (fr % 4) .. + 3
-#pragma unroll
-    for (int d = 0; d < DT; d++)
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
-            const int r = 32 * kh + 16 * hh + 4 * fg + (fr >> 2);
-            const int c = min(2 * d + ((fr & 3) >> 1), dvec - 1);
-            voff[d][hh] = blk_halfs + 8 * at_chunk_pos(r, c, dvec) + 4 * (fr & 1);
-        }
+    for (int d = 0; d < DT; d++) {
+        const int r = 32 * kh + 4 * fg + (fr >> 2);
+        const int c = min(2 * d + ((fr & 3) >> 1), dvec - 1);
+        voff[d] = blk_halfs + 8 * at_chunk_pos(r, c, dvec) + 4 * (fr & 1);
+    }
+    // with a fixed unswizzled row length the value fragments of all tiles inside head_dim are 32 bytes apart
+    constexpr bool VIMM = DC != 0 && DC != 64 && DC != 128;
+    constexpr int DTL = DC ? (DC + 15) / 16 : DT; // output tiles that hold a column of head_dim
     for (int it = 0; it < nkb; it++) {      // ring position `it` holds key block kb_lo + it
         const int kb = kb_lo + it;
         const int k0 = kb * AT_BK;
@@ -218,16 +248,52 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
         issue_loads_at(it + STAGES - 1, min(kb + STAGES - 1, last));
         const half_t *st = ring + (it % STAGES) * (2 * blk_halfs);
 
-        // S = Q K^T for this wavefront's 16 rows and its 32 keys of the block (key tiles 2 kh, 2 kh + 1)
-        float4_t S[2];
+        // S = Q K^T for this wavefront's 16 rows and its 32 keys of the block (key tiles 2 kh, 2 kh + 1): all key
+        // fragments are requested before the first MFMA (one trip to LDS, not one per fragment), and the two
+        // tiles' chains of dependent MFMAs alternate
+        half8_t fk[2][KK];
 #pragma unroll
-        for (int b2 = 0; b2 < 2; b2++) {
-            S[b2] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int b2 = 0; b2 < 2; b2++)
 #pragma unroll
-            for (int kk = 0; kk < KK; kk++) {
-                const half8_t fk = __builtin_bit_cast(half8_t, *(const uint4_t *)(st + koff[b2][kk]));
-                S[b2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fk, fq[kk], S[b2], 0, 0, 0);
-            }
+            for (int kk = 0; kk < KK; kk++) fk[b2][kk] = __builtin_bit_cast(half8_t, *(const uint4_t *)(st + koff[kk] + b2 * tile_halfs));
+        __builtin_amdgcn_sched_barrier(0);
+        float4_t S[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++)
+#pragma unroll
+            for (int b2 = 0; b2 < 2; b2++) S[b2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fk[b2][kk], fq[kk], S[b2], 0, 0, 0);
+        // The value fragments of O += P V do not depend on the scores: they are requested here and awaited after
+        // the softmax arithmetic, which hides their trip.  The transposing reads are issued from assembly: as a
+        // builtin the compiler orders them after every outstanding load into LDS (vmcnt(0)), which would drain
+        // the ring on every step.  Every tile is read and multiplied, also one wholly past head_dim (the clamped
+        // addresses stay inside the block, its columns are never stored).
+        const uint32_t st_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const half_t *)st;
+        uint64_t fv[DT][2];
+        if constexpr (DC != 0) {
+            // a pair of tiles: two address registers (the same one twice, VIMM) and immediate offsets; an odd count
+            // reads its last tile twice
+            constexpr int TB2 = 2 * 128 * (DC / 8); // bytes between the two halves of the value rows
+            constexpr int VS = VIMM ? 32 : 0;       // bytes from a tile to the next
+#define RT_AT_PAIR(d0)                                                                                                         \
+    if constexpr (DTL > d0) {                                                                                                  \
+        constexpr int d1 = d0 + 1 < DTL ? d0 + 1 : d0;                                                                         \
+        at_tr_read4<VS * d0, VS * d0 + TB2, VS * d1, VS * d1 + TB2>(fv[d0][0], fv[d0][1], fv[d0 + 1][0], fv[d0 + 1][1],        \
+                                                                    st_addr + 2 * voff[VIMM ? 0 : d0], st_addr + 2 * voff[VIMM ? 0 : d1]); \
+    }
+            RT_AT_PAIR(0)
+            RT_AT_PAIR(2)
+            RT_AT_PAIR(4)
+            RT_AT_PAIR(6)
+#undef RT_AT_PAIR
+        } else {
+#pragma unroll
+            for (int d0 = 0; d0 < DT; d0 += 2)
+                asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %5\n\t"
+                             "ds_read_b64_tr_b16 %2, %6\n\tds_read_b64_tr_b16 %3, %7"
+                             : "=&v"(fv[d0][0]), "=&v"(fv[d0][1]), "=&v"(fv[d0 + 1][0]), "=&v"(fv[d0 + 1][1])
+                             : "v"(st_addr + 2 * voff[d0]), "v"(st_addr + 2 * (voff[d0] + tile_halfs)),
+                               "v"(st_addr + 2 * voff[d0 + 1]), "v"(st_addr + 2 * (voff[d0 + 1] + tile_halfs))
+                             : "memory");
         }
         // scale, mask, bounds; then the row maximum over the wavefront's keys.  Only a block that
         // crosses the end of the keys or the causal diagonal of this wavefront's rows needs the
@@ -282,27 +348,20 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
 #pragma unroll
             for (int d = 0; d < DT; d++) acc[d] *= alpha;
         }
-        // O += P V over this wavefront's 32 keys; tiles wholly past head_dim are never stored.
-        // The transposing reads are issued from assembly, in groups that end with their own wait:
-        // as a builtin the compiler orders them after every outstanding load into LDS (vmcnt(0)),
-        // which would drain the ring on every step.
-        const uint32_t st_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const half_t *)st;
+        // O += P V over this wavefront's 32 keys.  The wait names every fragment register, so nothing that uses
+        // one can be placed before it.
+        constexpr int DTU = DTL; // tiles read and multiplied
 #pragma unroll
-        for (int d0 = 0; d0 < DT; d0 += 2) {
-            if (16 * d0 < g.D) { // uniform
-                uint64_t v00, v01, v10, v11;
-                asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %5\n\t"
-                             "ds_read_b64_tr_b16 %2, %6\n\tds_read_b64_tr_b16 %3, %7\n\ts_waitcnt lgkmcnt(0)"
-                             : "=&v"(v00), "=&v"(v01), "=&v"(v10), "=&v"(v11)
-                             : "v"(st_addr + 2 * voff[d0][0]), "v"(st_addr + 2 * voff[d0][1]),
-                               "v"(st_addr + 2 * voff[d0 + 1][0]), "v"(st_addr + 2 * voff[d0 + 1][1])
-                             : "memory");
-                typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
-                acc[d0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, u64x2_t{v00, v01}), fp, acc[d0], 0, 0, 0);
-                if (16 * (d0 + 1) < g.D)
-                    acc[d0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, u64x2_t{v10, v11}), fp, acc[d0 + 1], 0, 0, 0);
-            }
+        for (int d0 = 0; d0 < DTU; d0 += 2) {
+            if (d0 == 0)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fv[d0][0]), "+v"(fv[d0][1]), "+v"(fv[d0 + 1][0]), "+v"(fv[d0 + 1][1])::"memory");
+            else
+                asm volatile("" : "+v"(fv[d0][0]), "+v"(fv[d0][1]), "+v"(fv[d0 + 1][0]), "+v"(fv[d0 + 1][1])::"memory");
         }
+        typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int d = 0; d < DTU; d++)
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, u64x2_t{fv[d][0], fv[d][1]}), fp, acc[d], 0, 0, 0);
         // block kb + 1 has landed for everybody, and nobody reads block kb's stage any more
         publish(std::integral_constant<int, STAGES - 2>{});
     }
@@ -356,7 +415,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
 #pragma unroll
         for (int d = 0; d < DT; d++) {
             const int c = 16 * d + 4 * fg;
-            if (c < g.D) { // head_dim % 8 == 0 and c % 4 == 0: a group of four is inside or outside as a whole
+            if (c < D) { // head_dim % 8 == 0 and c % 4 == 0: a group of four is inside or outside as a whole
                 const half_t o4[4] = {(half_t)(acc[d][0] * inv), (half_t)(acc[d][1] * inv), (half_t)(acc[d][2] * inv),
                                       (half_t)(acc[d][3] * inv)};
                 *(uint64_t *)(op + c) = *(const uint64_t *)o4;
@@ -558,17 +617,17 @@ static uint64_t attention_decode_workspace_bytes(const rt_attention_desc &d) {
     return (uint64_t)d.batch * d.heads * attention_decode_splits(d) * AD_PSTRIDE * sizeof(float);
 }
 
-template <int DP, bool MASK> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
-    constexpr int STAGES = DP <= 96 ? 4 : 3;
+template <int DP, bool MASK, int DC> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
+    constexpr int STAGES = at_stages(DP);
     // the ring of packed key + value blocks; the merge of the key halves reuses it
     const size_t ring = (size_t)STAGES * 2 * AT_BK * g.D * sizeof(half_t);
     const size_t merge = (size_t)4 * (2 + 4 * (DP / 16)) * 64 * sizeof(float);
     const size_t lds = ring > merge ? ring : merge;
     if (lds > 48 * 1024) {
-        if (const hipError_t e = ensure_lds_limit<&attention_kernel<DP, MASK>>(); e != hipSuccess) return e;
+        if (const hipError_t e = ensure_lds_limit<&attention_kernel<DP, MASK, DC>>(); e != hipSuccess) return e;
     }
     const unsigned qb = (unsigned)((g.q_len + AT_BQ - 1) / AT_BQ);
-    hipLaunchKernelGGL((attention_kernel<DP, MASK>), dim3(qb, (unsigned)stacks, (unsigned)g.splits), dim3(AT_THREADS), lds, st, g);
+    hipLaunchKernelGGL((attention_kernel<DP, MASK, DC>), dim3(qb, (unsigned)stacks, (unsigned)g.splits), dim3(AT_THREADS), lds, st, g);
     if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (g.splits > 1) {
         hipLaunchKernelGGL((attention_merge_kernel<DP>), dim3(qb, (unsigned)stacks), dim3(256), 0, st, g);
@@ -577,8 +636,10 @@ template <int DP, bool MASK> static hipError_t launch_attention_dm(const AttnArg
     return hipSuccess;
 }
 
-template <int DP> static hipError_t launch_attention_dp(const AttnArgs &g, int stacks, hipStream_t st) {
-    return g.mask ? launch_attention_dm<DP, true>(g, stacks, st) : launch_attention_dm<DP, false>(g, stacks, st);
+// the kernel built for this head_dim (Whisper 64, Phi-2 80, Phi-3 96, Llama-class 128), else the one that takes it as an argument
+template <int DP, int DC> static hipError_t launch_attention_dp(const AttnArgs &g, int stacks, hipStream_t st) {
+    if (g.D == DC) return g.mask ? launch_attention_dm<DP, true, DC>(g, stacks, st) : launch_attention_dm<DP, false, DC>(g, stacks, st);
+    return g.mask ? launch_attention_dm<DP, true, 0>(g, stacks, st) : launch_attention_dm<DP, false, 0>(g, stacks, st);
 }
 
 static int attention_dp(int head_dim) { return head_dim <= 64 ? 64 : (head_dim <= 96 ? 96 : 128); }
@@ -635,9 +696,10 @@ hipError_t launch_attention(const rt_attention_desc &d, const void *q, const voi
         hipLaunchKernelGGL(attention_decode_merge_kernel, dim3((unsigned)stacks), dim3(128), 0, stream, g);
         return hipGetLastError();
     }
-    if (d.head_dim <= 64) return launch_attention_dp<64>(g, (int)stacks, stream);
-    if (d.head_dim <= 96) return launch_attention_dp<96>(g, (int)stacks, stream);
-    return launch_attention_dp<128>(g, (int)stacks, stream);
+    if (d.head_dim <= 64) return launch_attention_dp<64, 64>(g, (int)stacks, stream);
+    if (d.head_dim == 80) return launch_attention_dp<96, 80>(g, (int)stacks, stream);
+    if (d.head_dim <= 96) return launch_attention_dp<96, 96>(g, (int)stacks, stream);
+    return launch_attention_dp<128, 128>(g, (int)stacks, stream);
 }
 
 } // namespace rt
