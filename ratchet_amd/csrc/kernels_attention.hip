@@ -122,8 +122,22 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int qt = wave & 3, kh = wave >> 2;
     const int fr = lane & 15, fg = lane >> 4;
-    const int q0 = blockIdx.x * AT_BQ;
-    const int bh = blockIdx.y, b = bh / g.heads, h = bh - b * g.heads;
+    // Which (query block, head, split) this workgroup takes.  Workgroups go to the eight XCDs round-robin by their
+    // linear number; taken as it comes, the query blocks of one head would land on eight XCDs and every one of the
+    // eight L2s would fetch that head's keys and values.  When the grid divides by eight, XCD x instead takes the
+    // x-th eighth of the work items in (split, head, query block) order: all query blocks of a head share an L2.
+    uint32_t qbi = blockIdx.x, bhi = blockIdx.y, spi = blockIdx.z;
+    {
+        const uint32_t total = gridDim.x * gridDim.y * gridDim.z;
+        if ((total & 7u) == 0) {
+            const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+            const uint32_t w = (lin & 7u) * (total >> 3) + (lin >> 3);
+            const uint32_t wy = w / gridDim.x;
+            qbi = w - wy * gridDim.x, spi = wy / gridDim.y, bhi = wy - spi * gridDim.y;
+        }
+    }
+    const int q0 = (int)qbi * AT_BQ;
+    const int bh = (int)bhi, b = bh / g.heads, h = bh - b * g.heads;
     const half_t *Q = g.Q + b * g.q_bs + h * g.q_hs;
     const half_t *K = g.K + b * g.k_bs + h * g.k_hs;
     const half_t *V = g.V + b * g.v_bs + h * g.v_hs;
@@ -212,7 +226,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     if (g.causal) k_end = max(0, min(g.kv_len, q0 + AT_BQ + off));
     const int nkb_all = (k_end + AT_BK - 1) / AT_BK;
     // this workgroup's share of the key blocks: [kb_lo, kb_hi), an even split over gridDim.z
-    const int split = blockIdx.z;
+    const int split = (int)spi;
     const int kb_lo = (int)((int64_t)nkb_all * split / g.splits), kb_hi = (int)((int64_t)nkb_all * (split + 1) / g.splits);
     const int nkb = kb_hi - kb_lo;
     const int last = max(kb_hi - 1, 0);
@@ -401,7 +415,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     if (g.splits > 1) {
         // this workgroup saw only its share of the keys: hand (m, l, O) of every row to the merge kernel
         // (rows past q_len are never merged: a decode step has one live row of 64)
-        float *pr = g.partial + ((((size_t)blockIdx.y * gridDim.x + blockIdx.x) * g.splits + split) * AT_BQ + 16 * qt + fr) * (4 + DP);
+        float *pr = g.partial + ((((size_t)bhi * gridDim.x + qbi) * g.splits + split) * AT_BQ + 16 * qt + fr) * (4 + DP);
         if (qrow < g.q_len) {
             if (fg == 0) pr[0] = m_run, pr[1] = l_run;
 #pragma unroll
