@@ -181,19 +181,23 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
         ldst[i] = (lval[i] ? blk_halfs : 0) + 512 * jj;
     }
     // block `src_kb` into the stage of ring position `pos_kb` (they differ only past the end).  A block that lies
-    // wholly inside the keys is addressed as a uniform base (the block's first row: scalar arithmetic) plus the
-    // lane's fixed 32-bit byte offset inside a block, so a load costs no vector instruction beside itself.
-    uint32_t lofs[NI];     // byte offset of the lane's chunk from the block's first row
+    // wholly inside the keys is addressed as the lane's pointer into block 0 plus the block's byte offset, one
+    // scalar multiplication (the launcher keeps a head's keys and values within 2^32 bytes) and one vector addition.
+    const uint8_t *lptr[NI]; // the lane's chunk in block 0
+    uint32_t lstep[NI];      // bytes from a block to the next (uniform)
 #pragma unroll
-    for (int i = 0; i < NI; i++) lofs[i] = ((uint32_t)lrow[i] * (uint32_t)(lval[i] ? g.v_rs : g.k_rs) + lcol[i]) * 2u;
+    for (int i = 0; i < NI; i++) {
+        const uint32_t rs = (uint32_t)(lval[i] ? g.v_rs : g.k_rs);
+        lptr[i] = (const uint8_t *)(lval[i] ? V : K) + (size_t)(((uint32_t)lrow[i] * rs + lcol[i]) * 2u);
+        lstep[i] = (uint32_t)AT_BK * rs * 2u;
+    }
     auto issue_loads_at = [&](int pos_kb, int src_kb) {
         half_t *st = ring + (pos_kb % STAGES) * (2 * blk_halfs);
         const int k0 = src_kb * AT_BK;
         if (k0 + AT_BK <= g.kv_len) { // uniform
-            const uint8_t *kb0 = (const uint8_t *)(K + (int64_t)k0 * g.k_rs), *vb0 = (const uint8_t *)(V + (int64_t)k0 * g.v_rs);
 #pragma unroll
             for (int i = 0; i < NI; i++)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)((lval[i] ? vb0 : kb0) + lofs[i]),
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(lptr[i] + (size_t)((uint32_t)src_kb * lstep[i])),
                                                  (__attribute__((address_space(3))) void *)(st + ldst[i]), 16, 0, 0);
             return;
         }
@@ -227,7 +231,8 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     const int nkb_all = (k_end + AT_BK - 1) / AT_BK;
     // this workgroup's share of the key blocks: [kb_lo, kb_hi), an even split over gridDim.z
     const int split = (int)spi;
-    const int kb_lo = (int)((int64_t)nkb_all * split / g.splits), kb_hi = (int)((int64_t)nkb_all * (split + 1) / g.splits);
+    int kb_lo = 0, kb_hi = nkb_all;
+    if (g.splits > 1) kb_lo = (int)((uint32_t)(nkb_all * split) / (uint32_t)g.splits), kb_hi = (int)((uint32_t)(nkb_all * (split + 1)) / (uint32_t)g.splits);
     const int nkb = kb_hi - kb_lo;
     const int last = max(kb_hi - 1, 0);
     // prologue: the first STAGES - 1 blocks requested (an index past the end repeats the last block, so
@@ -255,7 +260,12 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     // with a fixed unswizzled row length the value fragments of all tiles inside head_dim are 32 bytes apart
     constexpr bool VIMM = DC != 0 && DC != 64 && DC != 128;
     constexpr int DTL = DC ? (DC + 15) / 16 : DT; // output tiles that hold a column of head_dim
-    for (int it = 0; it < nkb; it++) {      // ring position `it` holds key block kb_lo + it
+    // One step: ring position `it` holds key block kb_lo + it.  LEAN: the block crosses neither the end of the keys nor
+    // the causal diagonal of this wavefront's rows, there is no mask tensor and the scale is positive, so the step
+    // carries none of the tests for those (a wavefront issues an instruction every four cycles at best, whatever its
+    // kind: the scalar bookkeeping of a step costs as much time as its vector arithmetic).
+    auto step = [&](int it, auto lean_c) {
+        constexpr bool LEAN = decltype(lean_c)::value;
         const int kb = kb_lo + it;
         const int k0 = kb * AT_BK;
         // the stage the previous step used is free (everybody passed the barrier that ended it)
@@ -313,10 +323,10 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
         // crosses the end of the keys or the causal diagonal of this wavefront's rows needs the
         // per-element tests (uniform).
         const int kw0 = k0 + 32 * kh; // first of this wavefront's keys
-        const bool edge = kw0 + 32 > g.kv_len || (g.causal && kw0 + 31 > q0 + 16 * qt + off);
+        const bool edge = !LEAN && (kw0 + 32 > g.kv_len || (g.causal && kw0 + 31 > q0 + 16 * qt + off));
         // Fast path (scale > 0, no mask, no edge): the maximum is taken on the raw scores and the scale
         // is folded into the exponent's argument, exp2(S * c - m).
-        const bool raw = !MASK && !edge && g.scale_log2e > 0.f; // uniform
+        const bool raw = LEAN || (!MASK && !edge && g.scale_log2e > 0.f); // uniform
         float bmax = -INFINITY;
         if (raw) {
 #pragma unroll
@@ -378,6 +388,19 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
             acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, u64x2_t{fv[d][0], fv[d][1]}), fp, acc[d], 0, 0, 0);
         // block kb + 1 has landed for everybody, and nobody reads block kb's stage any more
         publish(std::integral_constant<int, STAGES - 2>{});
+    };
+    // the leading blocks of this wavefront's share that are lean: kw0 + 32 <= kv_len, and causal: kw0 + 31 <= first row + off
+    int n_lean = 0;
+    if (!MASK && g.scale_log2e > 0.f) {
+        auto blocks_upto = [](int num) { return num < 0 ? 0 : num / AT_BK + 1; }; // block numbers kb with AT_BK kb <= num
+        int n = blocks_upto(g.kv_len - 32 - 32 * kh);
+        if (g.causal) n = min(n, blocks_upto(q0 + 16 * qt + off - 31 - 32 * kh));
+        n_lean = max(0, min(n - kb_lo, nkb));
+    }
+    {
+        int it = 0;
+        for (; it < n_lean; it++) step(it, std::true_type{});
+        for (; it < nkb; it++) step(it, std::false_type{});
     }
     // no load may land in LDS once the merge below reuses it
     asm volatile("" ::: "memory");
