@@ -53,8 +53,7 @@ struct AttnArgs {
     float *partial;     // [stack][query block][split][64 rows][4 + DP]: running maximum, sum, two unused, unnormalised output
 };
 
-constexpr int AT_THREADS = 512, AT_BQ = 64, AT_BK = 64;
-constexpr int AT_WAVES = AT_THREADS / 64;
+constexpr int AT_BQ = 64, AT_BK = 64; // query rows of a workgroup; keys of a block of the eight-wavefront kernel (the unit the split heuristic counts in)
 constexpr float kLog2e = 1.4426950408889634f;
 
 // position (in 16-byte chunks) of chunk c of row r inside a packed block of rows of dvec chunks
@@ -88,7 +87,8 @@ __device__ __forceinline__ float at_groups_sum(float v) {
     return __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
 }
 
-constexpr int at_stages(int dp) { return dp <= 96 ? 4 : 3; } // stages of the key / value ring
+// stages of the key / value ring: blocks of 32 nkq keys, at most 160 KB
+constexpr int at_stages(int dp, int nkq) { return nkq == 4 ? 3 : (dp <= 96 ? 4 : 3); }
 
 // four transposing reads at two addresses with immediate offsets; nothing waits here
 template <int O0, int O1, int O2, int O3>
@@ -104,18 +104,26 @@ __device__ __forceinline__ void at_tr_read4(uint64_t &v0, uint64_t &v1, uint64_t
 // kernel is built for one (64, 80, 96, 128), else 0 and head_dim is the argument's: with a constant row length the
 // fragment addresses inside a stage differ by constants, which the LDS instructions carry as immediate offsets, so
 // a block costs three address additions instead of eighteen.
-// Eight wavefronts: wavefront (qt, kh) owns query tile qt (16 rows) and half kh (32 keys) of every
-// key block, with its own running maximum, sum and output; the two halves of a row are merged
-// through LDS at the end.  Two wavefronts per SIMD hide each other's latencies.
-template <int DP, bool MASK, int DC>
-__global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
+// 4 NKQ wavefronts: wavefront (qt, kh) owns query tile qt (16 rows) and part kh (32 keys) of every block of
+// 32 NKQ keys, with its own running maximum, sum and output; the NKQ parts of a row are merged through LDS at the
+// end.  NKQ = 2: eight wavefronts, blocks of 64 keys.  NKQ = 4: sixteen wavefronts, blocks of 128 keys; a wavefront
+// issues an instruction every four cycles at best and a step is some 130 of them whatever their kind, so with two
+// wavefronts per SIMD the vector unit is busy a third of the time: four per SIMD, each taking a quarter of a
+// block twice as long, do the same work in the same number of instructions per wavefront and half as many steps.
+// It needs the registers of a wavefront to stay within 128 and three stages of 128 keys within the LDS
+// (head_dim up to 96).
+template <int DP, bool MASK, int DC, int NKQ>
+__global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
+    static_assert(NKQ == 2 || (NKQ == 4 && DP <= 96), "eight wavefronts, or sixteen for head_dim up to 96");
+    constexpr int BK = 32 * NKQ, WAVES = 4 * NKQ; // keys of a block; wavefronts
     static_assert(DC == 0 || (DC % 8 == 0 && DC <= DP && DC > DP - 32), "a fixed head_dim belongs to its padded size");
     constexpr int KK = DP / 32;             // MFMA steps over head_dim
     constexpr int DT = DP / 16;             // 16-column tiles of the output
-    // load instructions per wavefront per block: a block is 2 * dvec instructions (64 chunks each,
-    // keys then values); instruction j belongs to wavefront j % 8, surplus ones repeat the last
-    constexpr int NI = (2 * (DP / 8) + AT_WAVES - 1) / AT_WAVES;
-    constexpr int STAGES = at_stages(DP);
+    // load instructions per wavefront per block: a block is 2 ipo instructions (64 chunks each, ipo = dvec NKQ / 2
+    // for the keys, then as many for the values); instruction j belongs to wavefront j % WAVES, surplus ones
+    // repeat the last
+    constexpr int NI = ((DP / 8) * NKQ + WAVES - 1) / WAVES;
+    constexpr int STAGES = at_stages(DP, NKQ);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int t = threadIdx.x, lane = t & 63;
@@ -146,7 +154,8 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     const int dvec = D >> 3;                // 16-byte chunks per row (head_dim % 8 == 0)
     const int off = g.kv_len - g.q_len;     // causal: query i sees keys <= i + off
     const uint4_t zero4 = {0u, 0u, 0u, 0u};
-    const int blk_halfs = AT_BK * D;        // one packed block of keys (or values)
+    const int blk_halfs = BK * D;           // one packed block of keys (or values)
+    const int ipo = dvec * NKQ / 2;         // load instructions per operand and block
     half_t *ring = (half_t *)smem;          // [STAGES][keys | values][64 rows][D]
 
     // this wavefront's Q fragments: row q0 + 16 qt + fr, head_dim 32 kk + 8 fg .. + 7 (zero past head_dim)
@@ -170,9 +179,9 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     int ldst[NI];          // LDS offset (halfs) of the instruction's 64 chunks inside a stage
 #pragma unroll
     for (int i = 0; i < NI; i++) {
-        const int j = min(wave + AT_WAVES * i, 2 * dvec - 1);   // surplus instructions repeat the block's last one
-        lval[i] = j >= dvec;
-        const int jj = lval[i] ? j - dvec : j;
+        const int j = min(wave + WAVES * i, 2 * ipo - 1);      // surplus instructions repeat the block's last one
+        lval[i] = j >= ipo;
+        const int jj = lval[i] ? j - ipo : j;
         const int q = 64 * jj + lane;
         lrow[i] = q / dvec;
         const int pos = q - lrow[i] * dvec;                        // position inside the row ...
@@ -189,12 +198,12 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     for (int i = 0; i < NI; i++) {
         const uint32_t rs = (uint32_t)(lval[i] ? g.v_rs : g.k_rs);
         lptr[i] = (const uint8_t *)(lval[i] ? V : K) + (size_t)(((uint32_t)lrow[i] * rs + lcol[i]) * 2u);
-        lstep[i] = (uint32_t)AT_BK * rs * 2u;
+        lstep[i] = (uint32_t)BK * rs * 2u;
     }
     auto issue_loads_at = [&](int pos_kb, int src_kb) {
         half_t *st = ring + (pos_kb % STAGES) * (2 * blk_halfs);
-        const int k0 = src_kb * AT_BK;
-        if (k0 + AT_BK <= g.kv_len) { // uniform
+        const int k0 = src_kb * BK;
+        if (k0 + BK <= g.kv_len) { // uniform
 #pragma unroll
             for (int i = 0; i < NI; i++)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(lptr[i] + (size_t)((uint32_t)src_kb * lstep[i])),
@@ -228,7 +237,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     // causal: key blocks wholly above the diagonal of this query block are never visited
     int k_end = g.kv_len;
     if (g.causal) k_end = max(0, min(g.kv_len, q0 + AT_BQ + off));
-    const int nkb_all = (k_end + AT_BK - 1) / AT_BK;
+    const int nkb_all = (k_end + BK - 1) / BK;
     // this workgroup's share of the key blocks: [kb_lo, kb_hi), an even split over gridDim.z
     const int split = (int)spi;
     int kb_lo = 0, kb_hi = nkb_all;
@@ -267,7 +276,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     auto step = [&](int it, auto lean_c) {
         constexpr bool LEAN = decltype(lean_c)::value;
         const int kb = kb_lo + it;
-        const int k0 = kb * AT_BK;
+        const int k0 = kb * BK;
         // the stage the previous step used is free (everybody passed the barrier that ended it)
         issue_loads_at(it + STAGES - 1, min(kb + STAGES - 1, last));
         const half_t *st = ring + (it % STAGES) * (2 * blk_halfs);
@@ -392,7 +401,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     // the leading blocks of this wavefront's share that are lean: kw0 + 32 <= kv_len, and causal: kw0 + 31 <= first row + off
     int n_lean = 0;
     if (!MASK && g.scale_log2e > 0.f) {
-        auto blocks_upto = [](int num) { return num < 0 ? 0 : num / AT_BK + 1; }; // block numbers kb with AT_BK kb <= num
+        auto blocks_upto = [](int num) { return num < 0 ? 0 : num / BK + 1; }; // block numbers kb with BK kb <= num
         int n = blocks_upto(g.kv_len - 32 - 32 * kh);
         if (g.causal) n = min(n, blocks_upto(q0 + 16 * qt + off - 31 - 32 * kh));
         n_lean = max(0, min(n - kb_lo, nkb));
@@ -408,10 +417,12 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
-    // merge the two key halves of every row: the kh = 1 wavefront hands (m, l, O) to its kh = 0 partner
-    // through LDS, lane to lane
-    float *ex = (float *)smem + (size_t)qt * (2 + 4 * DT) * 64 + lane; // [qt][2 + 4 DT][64 lanes]
-    if (kh == 1) {
+    // merge the key parts of every row: the kh > 0 wavefronts hand (m, l, O) to their kh = 0 partner through LDS,
+    // lane to lane
+    constexpr int EXW = (2 + 4 * DT) * 64; // floats one wavefront hands over
+    float *exb = (float *)smem + (size_t)qt * EXW + lane; // [kh - 1][qt][2 + 4 DT][64 lanes]
+    if (kh > 0) {
+        float *ex = exb + (size_t)(kh - 1) * 4 * EXW;
         ex[0] = m_run;
         ex[64] = l_run;
 #pragma unroll
@@ -420,18 +431,30 @@ __global__ __launch_bounds__(AT_THREADS) void attention_kernel(AttnArgs g) {
             for (int r = 0; r < 4; r++) ex[(2 + 4 * d + r) * 64] = acc[d][r];
     }
     __syncthreads();
-    if (kh == 1) return;
+    if (kh > 0) return;
     {
-        const float m1 = ex[0], l1 = ex[64];
-        const float m_new = fmaxf(m_run, m1);
+        float mp[NKQ - 1], lp[NKQ - 1];
+        float m_new = m_run;
+#pragma unroll
+        for (int p = 0; p < NKQ - 1; p++) {
+            mp[p] = exb[(size_t)p * 4 * EXW], lp[p] = exb[(size_t)p * 4 * EXW + 64];
+            m_new = fmaxf(m_new, mp[p]);
+        }
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float a0 = __builtin_amdgcn_exp2f(m_run - m_use), a1 = __builtin_amdgcn_exp2f(m1 - m_use);
-        l_run = l_run * a0 + l1 * a1;
+        const float a0 = __builtin_amdgcn_exp2f(m_run - m_use);
+        l_run *= a0;
+#pragma unroll
+        for (int d = 0; d < DT; d++) acc[d] *= a0;
+#pragma unroll
+        for (int p = 0; p < NKQ - 1; p++) {
+            const float ap = __builtin_amdgcn_exp2f(mp[p] - m_use);
+            l_run += lp[p] * ap;
+#pragma unroll
+            for (int d = 0; d < DT; d++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[d][r] += exb[(size_t)p * 4 * EXW + (2 + 4 * d + r) * 64] * ap;
+        }
         m_run = m_new; // what the sums and outputs are now relative to (a split launch hands it on)
-#pragma unroll
-        for (int d = 0; d < DT; d++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) acc[d][r] = acc[d][r] * a0 + ex[(2 + 4 * d + r) * 64] * a1;
     }
     // the row's sum over its four lanes, then O / l; lane (fr, fg) holds columns 16 d + 4 fg + r of row fr
     l_run = at_groups_sum(l_run);
@@ -654,23 +677,35 @@ static uint64_t attention_decode_workspace_bytes(const rt_attention_desc &d) {
     return (uint64_t)d.batch * d.heads * attention_decode_splits(d) * AD_PSTRIDE * sizeof(float);
 }
 
-template <int DP, bool MASK, int DC> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
-    constexpr int STAGES = at_stages(DP);
-    // the ring of packed key + value blocks; the merge of the key halves reuses it
-    const size_t ring = (size_t)STAGES * 2 * AT_BK * g.D * sizeof(half_t);
-    const size_t merge = (size_t)4 * (2 + 4 * (DP / 16)) * 64 * sizeof(float);
+template <int DP, bool MASK, int DC, int NKQ> static hipError_t launch_attention_k(const AttnArgs &g, int stacks, hipStream_t st) {
+    constexpr int STAGES = at_stages(DP, NKQ);
+    // the ring of packed key + value blocks; the merge of the key parts reuses it
+    const size_t ring = (size_t)STAGES * 2 * (32 * NKQ) * g.D * sizeof(half_t);
+    const size_t merge = (size_t)(NKQ - 1) * 4 * (2 + 4 * (DP / 16)) * 64 * sizeof(float);
     const size_t lds = ring > merge ? ring : merge;
     if (lds > 48 * 1024) {
-        if (const hipError_t e = ensure_lds_limit<&attention_kernel<DP, MASK, DC>>(); e != hipSuccess) return e;
+        if (const hipError_t e = ensure_lds_limit<&attention_kernel<DP, MASK, DC, NKQ>>(); e != hipSuccess) return e;
     }
     const unsigned qb = (unsigned)((g.q_len + AT_BQ - 1) / AT_BQ);
-    hipLaunchKernelGGL((attention_kernel<DP, MASK, DC>), dim3(qb, (unsigned)stacks, (unsigned)g.splits), dim3(AT_THREADS), lds, st, g);
+    hipLaunchKernelGGL((attention_kernel<DP, MASK, DC, NKQ>), dim3(qb, (unsigned)stacks, (unsigned)g.splits), dim3(256 * NKQ), lds, st, g);
     if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (g.splits > 1) {
         hipLaunchKernelGGL((attention_merge_kernel<DP>), dim3(qb, (unsigned)stacks), dim3(256), 0, st, g);
         return hipGetLastError();
     }
     return hipSuccess;
+}
+
+// keys from which a launch in one pass takes the sixteen-wavefront kernel (head_dim up to 96).  32 heads x 512 queries x
+// head_dim 80, eight / sixteen wavefronts: 512 keys 10.0 / 10.7 us, 1024: 15.1 / 15.1, 1536: 21.3 / 20.1, 4096: 43.6 / 41.6;
+// 6 heads x 1500 x 1500 x 64 (Whisper): 17.8 / 15.8; 32 x 2048 x 2048 x 96 causal: 78.3 / 71.8
+RT_TUNABLE(g_attention_wide_from, 1280);
+
+template <int DP, bool MASK, int DC> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
+    if constexpr (DP <= 96) {
+        if (g.splits == 1 && g.kv_len >= g_attention_wide_from) return launch_attention_k<DP, MASK, DC, 4>(g, stacks, st);
+    }
+    return launch_attention_k<DP, MASK, DC, 2>(g, stacks, st);
 }
 
 // the kernel built for this head_dim (Whisper 64, Phi-2 80, Phi-3 96, Llama-class 128), else the one that takes it as an argument

@@ -184,6 +184,31 @@ def test_causal_and_masks(device, oracle):
 
 
 @gpu
+def test_long_key_streams_one_pass(device, oracle):
+    """From 1280 keys a launch in one pass (128 workgroups or more, so the keys are not shared out) runs sixteen
+    wavefronts over blocks of 128 keys for head_dim up to 96: key counts on and off a block, every masking mode, a late
+    dominant key, and head_dim 128, which stays with eight wavefronts."""
+    rng = np.random.default_rng(14)
+    for i, (B, H, Lq, Lk, D) in enumerate([(1, 64, 128, 1280, 80), (1, 64, 70, 1301, 64), (2, 32, 128, 1535, 96), (1, 128, 64, 1408, 40),
+                                           (1, 64, 128, 1300, 128)]):
+        q, k, v = rand_qkv(rng, B, H, Lq, Lk, D)
+        assert_close(run(device, q, k, v), oracle.attention(q, k, v), ("plain", i))
+        got = run(device, q, k, v, causal=True)
+        assert_close(got, oracle.attention(q, k, v, causal=True), ("causal", i))
+        tri = np.triu(np.full((Lq, Lk), -np.inf, np.float32), 1 + Lk - Lq)
+        np.testing.assert_allclose(run(device, q, k, v, mask=tri).astype(np.float32), got.astype(np.float32), rtol=4e-3, atol=1e-3)
+        mask = (rng.standard_normal((Lq, Lk)) * 2).astype(np.float32)
+        mask[rng.random((Lq, Lk)) < 0.3] = -np.inf
+        mask[:, 0] = 0
+        assert_close(run(device, q, k, v, mask=mask, scale=0.25), oracle.attention(q, k, v, mask=mask, scale=0.25), ("mask", i))
+    q, k, v = rand_qkv(rng, 1, 128, 64, 1400, 64)
+    q[..., 0], k[..., 0] = 30, 0
+    k[:, :, 1390, 0] = 30                      # key 1390 scores 900 above the rest: it arrives in the last block, fourth part
+    got = run(device, q, k, v, scale=1.0)
+    assert np.array_equal(got, np.broadcast_to(v[:, :, 1390:1391], q.shape))
+
+
+@gpu
 def test_softmax_extremes(device, oracle):
     """Scores far apart (one key takes everything) and large scores that would overflow exp without
     the running maximum; a change of the maximum late in the key stream rescales what was summed."""
