@@ -136,8 +136,9 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
     // x-th eighth of the work items in (split, head, query block) order: all query blocks of a head share an L2.
     uint32_t qbi = blockIdx.x, bhi = blockIdx.y, spi = blockIdx.z;
     {
-        const uint32_t total = gridDim.x * gridDim.y * gridDim.z;
-        if ((total & 7u) == 0) {
+        const uint64_t total64 = (uint64_t)gridDim.x * gridDim.y * gridDim.z;
+        if (total64 < (1u << 31) && (total64 & 7u) == 0) {
+            const uint32_t total = (uint32_t)total64;
             const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
             const uint32_t w = (lin & 7u) * (total >> 3) + (lin >> 3);
             const uint32_t wy = w / gridDim.x;

@@ -845,10 +845,19 @@ __global__ __launch_bounds__(NT_THREADS, 2) void gemm_nt_shortk_kernel(GemmNtArg
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wi = wave >> 1, wj = wave & 1;
     const int fr = lane & 15, fg = lane >> 4;
-    // blockIdx.x = strip * parts + part: the workgroups of a strip take its A tiles round-robin
-    const int parts = g.tiles_i, part = (int)(blockIdx.x % parts);
-    const int64_t j0 = (int64_t)(blockIdx.x / parts) * BN;
-    const int64_t s = blockIdx.y;
+    // Workgroups go to the eight XCDs round-robin by their linear number.  Taken as it comes, the strips of one stack
+    // land on all eight and every L2 fetches that stack's operands (3 x the operand bytes at 32 x [512 x 80] . [512 x 80]^T);
+    // when the grid divides by eight, XCD x takes the x-th eighth of the (stack, strip, part) items instead.
+    uint32_t bx = blockIdx.x, by = blockIdx.y;
+    if (const uint64_t total64 = (uint64_t)gridDim.x * gridDim.y; total64 < (1u << 31) && (total64 & 7u) == 0) {
+        const uint32_t total = (uint32_t)total64;
+        const uint32_t lin = blockIdx.x + gridDim.x * blockIdx.y, w = (lin & 7u) * (total >> 3) + (lin >> 3);
+        by = w / gridDim.x, bx = w - by * gridDim.x;
+    }
+    // bx = strip * parts + part: the workgroups of a strip take its A tiles round-robin
+    const int parts = g.tiles_i, part = (int)(bx % parts);
+    const int64_t j0 = (int64_t)(bx / parts) * BN;
+    const int64_t s = by;
     const int64_t a_el = (g.a_stack == 1 ? 0 : s) * g.a_bs, b_el = (g.b_stack == 1 ? 0 : s) * g.b_bs;
     const int kvecs = (int)(g.K >> 3);
     const uint4_t zero4 = {0u, 0u, 0u, 0u};
