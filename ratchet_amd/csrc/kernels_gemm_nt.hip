@@ -555,7 +555,11 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_dl_kernel(GemmNt
 // fragments (50 of their 153 vector instructions per K step), 43.2 us; this one 41.6: what is left is the
 // fold, four fused multiply-adds per MFMA, which the multiplying wavefronts cannot hand to anyone.
 // Rounding q * d to f16 (the reference's own shader does, ops/gemm.rs:547-548) would remove the fold, and was
-// measured: the outputs near zero then miss the 2e-2 tolerance (0.115).
+// measured: the outputs near zero then miss the 2e-2 tolerance (0.115).  The hi / lo form was built once more on this
+// pipeline (the loading wavefronts computing both tiles, two weight stages of hi and lo and four activation stages,
+// the multiplying wavefronts issuing MFMAs only): 57.1 us against this kernel's 44.3 in the same harness.  The lo tile
+// is subnormal f16 as a rule, which the matrix cores take at full speed (scaled into the normal range it ran the
+// same); the form doubles the weight fragments read from LDS and the stores of the loading wavefronts.
 //
 // Ring of four stages of (BM + BN) x 64 halves.  Loading wavefront, iteration j: request the codes of tile
 // j + 3 (registers, set (j + 3) % 4) and its activation rows (LDS-DMA into stage (j + 3) % 4, last read
@@ -618,8 +622,10 @@ __global__ __launch_bounds__(NT_THREADS + 64 * LW) void gemm_nt_q8w_kernel(GemmN
             for (int c = 0; c < LCHB; c++)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb[c] + k0),
                                                  (__attribute__((address_space(3))) void *)(st + (lw + c * LW) * 8 * NT_LDK), 16, 0, 0);
+            __builtin_amdgcn_sched_barrier(0); // the wait in widen_store counts the loads in this order
 #pragma unroll
             for (int c = 0; c < NA; c++) ra[slot][c] = *(const uint4_t *)(ga[c] + k0);
+            __builtin_amdgcn_sched_barrier(0);
         };
         auto widen_store = [&](int slot) __attribute__((always_inline)) {
             asm volatile("" ::: "memory");
