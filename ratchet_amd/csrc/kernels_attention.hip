@@ -73,7 +73,9 @@ __device__ __forceinline__ constexpr int at_waitcnt(int n) { return 0x0070 | (n 
 __device__ __forceinline__ float at_groups_max(float v) {
     const uint32_t u = __builtin_bit_cast(uint32_t, v);
     const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    const float w = fmaxf(__builtin_bit_cast(float, (uint32_t)a[0]), __builtin_bit_cast(float, (uint32_t)a[1]));
+    // the instruction itself: fmaxf() of values that come out of a bit cast first quiets each of them (two more instructions)
+    float w;
+    asm("v_max_f32 %0, %1, %2" : "=v"(w) : "v"((uint32_t)a[0]), "v"((uint32_t)a[1]));
     const uint32_t x = __builtin_bit_cast(uint32_t, w);
     const auto b = __builtin_amdgcn_permlane32_swap(x, x, false, false);
     return fmaxf(__builtin_bit_cast(float, (uint32_t)b[0]), __builtin_bit_cast(float, (uint32_t)b[1]));
@@ -98,6 +100,10 @@ __device__ __forceinline__ void at_tr_read4(uint64_t &v0, uint64_t &v1, uint64_t
                  : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
                  : "v"(a0), "v"(a1), "n"(O0), "n"(O1), "n"(O2), "n"(O3)
                  : "memory");
+}
+
+template <int O0, int O1> __device__ __forceinline__ void at_tr_read2(uint64_t &v0, uint64_t &v1, uint32_t a0) {
+    asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4" : "=&v"(v0), "=&v"(v1) : "v"(a0), "n"(O0), "n"(O1) : "memory");
 }
 
 // DP: head_dim padded to a multiple of 32.  MASK: an additive mask tensor is present.  DC: head_dim itself when the
@@ -304,15 +310,15 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
         const uint32_t st_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const half_t *)st;
         uint64_t fv[DT][2];
         if constexpr (DC != 0) {
-            // a pair of tiles: two address registers (the same one twice, VIMM) and immediate offsets; an odd count
-            // reads its last tile twice
+            // a pair of tiles: two address registers (the same one twice, VIMM) and immediate offsets
             constexpr int TB2 = 2 * 128 * (DC / 8); // bytes between the two halves of the value rows
             constexpr int VS = VIMM ? 32 : 0;       // bytes from a tile to the next
 #define RT_AT_PAIR(d0)                                                                                                         \
-    if constexpr (DTL > d0) {                                                                                                  \
-        constexpr int d1 = d0 + 1 < DTL ? d0 + 1 : d0;                                                                         \
-        at_tr_read4<VS * d0, VS * d0 + TB2, VS * d1, VS * d1 + TB2>(fv[d0][0], fv[d0][1], fv[d0 + 1][0], fv[d0 + 1][1],        \
-                                                                    st_addr + 2 * voff[VIMM ? 0 : d0], st_addr + 2 * voff[VIMM ? 0 : d1]); \
+    if constexpr (DTL > d0 + 1) {                                                                                              \
+        at_tr_read4<VS * d0, VS * d0 + TB2, VS * (d0 + 1), VS * (d0 + 1) + TB2>(fv[d0][0], fv[d0][1], fv[d0 + 1][0], fv[d0 + 1][1], \
+                                                                                st_addr + 2 * voff[VIMM ? 0 : d0], st_addr + 2 * voff[VIMM ? 0 : d0 + 1]); \
+    } else if constexpr (DTL > d0) {                                                                                           \
+        at_tr_read2<VS * d0, VS * d0 + TB2>(fv[d0][0], fv[d0][1], st_addr + 2 * voff[VIMM ? 0 : d0]);                          \
     }
             RT_AT_PAIR(0)
             RT_AT_PAIR(2)
@@ -389,8 +395,10 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
         for (int d0 = 0; d0 < DTU; d0 += 2) {
             if (d0 == 0)
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fv[d0][0]), "+v"(fv[d0][1]), "+v"(fv[d0 + 1][0]), "+v"(fv[d0 + 1][1])::"memory");
-            else
+            else if (d0 + 1 < DTU)
                 asm volatile("" : "+v"(fv[d0][0]), "+v"(fv[d0][1]), "+v"(fv[d0 + 1][0]), "+v"(fv[d0 + 1][1])::"memory");
+            else
+                asm volatile("" : "+v"(fv[d0][0]), "+v"(fv[d0][1])::"memory");
         }
         typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
