@@ -106,7 +106,8 @@ template <int O0, int O1> __device__ __forceinline__ void at_tr_read2(uint64_t &
     asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4" : "=&v"(v0), "=&v"(v1) : "v"(a0), "n"(O0), "n"(O1) : "memory");
 }
 
-// DP: head_dim padded to a multiple of 32.  MASK: an additive mask tensor is present.  DC: head_dim itself when the
+// DP: head_dim padded to a multiple of 32.  MK: 0 no mask tensor; 1 an additive mask tensor, read from memory where it is
+// used; 2 the same, its [64 queries x 64 keys] block travelling through the ring with the keys and values (see below).  DC: head_dim itself when the
 // kernel is built for one (64, 80, 96, 128), else 0 and head_dim is the argument's: with a constant row length the
 // fragment addresses inside a stage differ by constants, which the LDS instructions carry as immediate offsets, so
 // a block costs three address additions instead of eighteen.
@@ -118,9 +119,16 @@ template <int O0, int O1> __device__ __forceinline__ void at_tr_read2(uint64_t &
 // block twice as long, do the same work in the same number of instructions per wavefront and half as many steps.
 // It needs the registers of a wavefront to stay within 128 and three stages of 128 keys within the LDS
 // (head_dim up to 96).
-template <int DP, bool MASK, int DC, int NKQ>
+// The mask tensor.  Read where it is used (eight loads per lane in the middle of a step, which the compiler has to
+// await with every load into LDS still in flight: the ring drains on every step, 25.7 us at 32 x 512 x 512 x 80 where
+// the causal flag takes 10.0) it is the slow path, yet a tensor is what the reference's callers pass
+// (phi3/attn.rs:148-151).  With rows of whole 16-byte vectors (MK == 2) the block's 64 x 64 mask values are two more
+// LDS-DMA instructions per wavefront and block, counted with the others, stored behind the values in the stage with
+// the row's 16-byte chunks XOR-swizzled like the keys', and read back as two vectors per lane.
+template <int DP, int MK, int DC, int NKQ>
 __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
-    static_assert(NKQ == 2 || (NKQ == 4 && DP <= 96), "eight wavefronts, or sixteen for head_dim up to 96");
+    constexpr bool MASK = MK != 0, MST = MK == 2;
+    static_assert(NKQ == 2 || (NKQ == 4 && DP <= 96 && !MST), "eight wavefronts, or sixteen for head_dim up to 96 (not with a staged mask)");
     constexpr int BK = 32 * NKQ, WAVES = 4 * NKQ; // keys of a block; wavefronts
     static_assert(DC == 0 || (DC % 8 == 0 && DC <= DP && DC > DP - 32), "a fixed head_dim belongs to its padded size");
     constexpr int KK = DP / 32;             // MFMA steps over head_dim
@@ -129,7 +137,8 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
     // for the keys, then as many for the values); instruction j belongs to wavefront j % WAVES, surplus ones
     // repeat the last
     constexpr int NI = ((DP / 8) * NKQ + WAVES - 1) / WAVES;
-    constexpr int STAGES = at_stages(DP, NKQ);
+    constexpr int NIM = MST ? 2 : 0;        // the mask block's instructions per wavefront (16 of 1 KB for f32, 8 for f16: the rest repeat the last)
+    constexpr int STAGES = MST ? 3 : at_stages(DP, NKQ);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int t = threadIdx.x, lane = t & 63;
@@ -162,6 +171,8 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
     const int off = g.kv_len - g.q_len;     // causal: query i sees keys <= i + off
     const uint4_t zero4 = {0u, 0u, 0u, 0u};
     const int blk_halfs = BK * D;           // one packed block of keys (or values)
+    const int mesz = g.mask_f32 ? 4 : 2, mcpr = BK * mesz / 16;            // mask: bytes per value, 16-byte chunks per row of a block
+    const int stage_halfs = 2 * blk_halfs + (MST ? AT_BQ * BK * mesz / 2 : 0); // keys, values (, mask)
     const int ipo = dvec * NKQ / 2;         // load instructions per operand and block
     half_t *ring = (half_t *)smem;          // [STAGES][keys | values][64 rows][D]
 
@@ -207,9 +218,33 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
         lptr[i] = (const uint8_t *)(lval[i] ? V : K) + (size_t)(((uint32_t)lrow[i] * rs + lcol[i]) * 2u);
         lstep[i] = (uint32_t)BK * rs * 2u;
     }
+    const uint8_t *mptr[MST ? NIM : 1]; // the lane's mask row
+    uint32_t mcol[MST ? NIM : 1];       // byte offset of its source chunk inside a block's columns
+    int mdst[MST ? NIM : 1];            // LDS offset (halfs) of the instruction's 64 chunks inside the mask block
+    if constexpr (MST) {
+#pragma unroll
+        for (int i = 0; i < NIM; i++) {
+            const int m = min(wave + WAVES * i, mcpr - 1);
+            const int c = 64 * m + lane, row = c / mcpr, pos = c - row * mcpr;
+            const int src = at_chunk_pos(row, pos, mcpr) - row * mcpr;
+            mptr[i] = (const uint8_t *)g.mask + (int64_t)min(q0 + row, g.q_len - 1) * g.mask_rs * mesz;
+            mcol[i] = 16u * (uint32_t)src;
+            mdst[i] = 512 * m;
+        }
+    }
     auto issue_loads_at = [&](int pos_kb, int src_kb) {
-        half_t *st = ring + (pos_kb % STAGES) * (2 * blk_halfs);
+        half_t *st = ring + (pos_kb % STAGES) * stage_halfs;
         const int k0 = src_kb * BK;
+        if constexpr (MST) {
+            // lane l of instruction m fills chunk 64 m + l of the mask block: row (64 m + l) / mcpr, and the source chunk the
+            // swizzle puts at that position; past the row's end (a last, partial block) the row's last chunk again
+#pragma unroll
+            for (int i = 0; i < NIM; i++) {
+                const uint32_t mo = min((uint32_t)(k0 * mesz) + mcol[i], (uint32_t)(g.mask_rs * mesz) - 16u);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(mptr[i] + mo),
+                                                 (__attribute__((address_space(3))) void *)(st + 2 * blk_halfs + mdst[i]), 16, 0, 0);
+            }
+        }
         if (k0 + BK <= g.kv_len) { // uniform
 #pragma unroll
             for (int i = 0; i < NI; i++)
@@ -230,7 +265,7 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
     // then everybody's have
     auto publish = [&](auto keep) {
         asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_waitcnt(at_waitcnt(decltype(keep)::value * NI));
+        __builtin_amdgcn_s_waitcnt(at_waitcnt(decltype(keep)::value * (NI + NIM)));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
@@ -258,7 +293,7 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
         for (int sidx = 0; sidx < STAGES - 1; sidx++) issue_loads_at(sidx, min(kb_lo + sidx, last));
     }
     const half_t *mrow = nullptr;
-    if constexpr (MASK) mrow = (const half_t *)g.mask; // indexed below by its own element type
+    if constexpr (MASK && !MST) mrow = (const half_t *)g.mask; // indexed below by its own element type
     if (nkb > 0) publish(std::integral_constant<int, STAGES - 2>{});
     // fragment addressing inside a stage (halfs).  Sixteen rows further down the swizzle repeats, so the second key
     // tile and the second half of the value rows are 16 dvec chunks away from the first.
@@ -286,7 +321,7 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
         const int k0 = kb * BK;
         // the stage the previous step used is free (everybody passed the barrier that ended it)
         issue_loads_at(it + STAGES - 1, min(kb + STAGES - 1, last));
-        const half_t *st = ring + (it % STAGES) * (2 * blk_halfs);
+        const half_t *st = ring + (it % STAGES) * stage_halfs;
 
         // S = Q K^T for this wavefront's 16 rows and its 32 keys of the block (key tiles 2 kh, 2 kh + 1): all key
         // fragments are requested before the first MFMA (one trip to LDS, not one per fragment), and the two
@@ -302,6 +337,26 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
         for (int kk = 0; kk < KK; kk++)
 #pragma unroll
             for (int b2 = 0; b2 < 2; b2++) S[b2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fk[b2][kk], fq[kk], S[b2], 0, 0, 0);
+        // this lane's mask values: row 16 qt + fr, keys 32 kh + 16 b2 + 4 fg .. + 3 of the block, one vector per key tile
+        float mvals[2][4];
+        if constexpr (MST) {
+            const uint8_t *mb = (const uint8_t *)(st + 2 * blk_halfs);
+            const int row = 16 * qt + fr;
+#pragma unroll
+            for (int b2 = 0; b2 < 2; b2++) {
+                if (g.mask_f32) { // uniform
+                    const float4_t mv = *(const float4_t *)(mb + 16 * at_chunk_pos(row, 8 * kh + 4 * b2 + fg, 16));
+#pragma unroll
+                    for (int r = 0; r < 4; r++) mvals[b2][r] = mv[r];
+                } else {
+                    const uint64_t raw = *(const uint64_t *)(mb + 16 * at_chunk_pos(row, 4 * kh + 2 * b2 + (fg >> 1), 8) + 8 * (fg & 1));
+                    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+                    const half4_t mh = __builtin_bit_cast(half4_t, raw);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) mvals[b2][r] = (float)mh[r];
+                }
+            }
+        }
         // The value fragments of O += P V do not depend on the scores: they are requested here and awaited after
         // the softmax arithmetic, which hides their trip.  The transposing reads are issued from assembly: as a
         // builtin the compiler orders them after every outstanding load into LDS (vmcnt(0)), which would drain
@@ -357,7 +412,9 @@ __global__ __launch_bounds__(256 * NKQ) void attention_kernel(AttnArgs g) {
                 for (int r = 0; r < 4; r++) {
                     const int key = kw0 + 16 * b2 + 4 * fg + r;
                     float s = S[b2][r] * g.scale_log2e;
-                    if constexpr (MASK) {
+                    if constexpr (MST) {
+                        s += mvals[b2][r] * kLog2e;
+                    } else if constexpr (MASK) {
                         const int64_t mi = (int64_t)min(qrow, g.q_len - 1) * g.mask_rs + min(key, g.kv_len - 1);
                         const float mv = g.mask_f32 ? ((const float *)mrow)[mi] : (float)mrow[mi];
                         s += mv * kLog2e;
@@ -686,17 +743,19 @@ static uint64_t attention_decode_workspace_bytes(const rt_attention_desc &d) {
     return (uint64_t)d.batch * d.heads * attention_decode_splits(d) * AD_PSTRIDE * sizeof(float);
 }
 
-template <int DP, bool MASK, int DC, int NKQ> static hipError_t launch_attention_k(const AttnArgs &g, int stacks, hipStream_t st) {
-    constexpr int STAGES = at_stages(DP, NKQ);
-    // the ring of packed key + value blocks; the merge of the key parts reuses it
-    const size_t ring = (size_t)STAGES * 2 * (32 * NKQ) * g.D * sizeof(half_t);
+template <int DP, int MK, int DC, int NKQ> static hipError_t launch_attention_k(const AttnArgs &g, int stacks, hipStream_t st) {
+    constexpr int STAGES = MK == 2 ? 3 : at_stages(DP, NKQ);
+    // the ring of packed key + value (+ mask) blocks; the merge of the key parts reuses it
+    const size_t stage = (size_t)2 * (32 * NKQ) * g.D * sizeof(half_t) + (MK == 2 ? (size_t)AT_BQ * (32 * NKQ) * (g.mask_f32 ? 4 : 2) : 0);
+    const size_t ring = STAGES * stage;
     const size_t merge = (size_t)(NKQ - 1) * 4 * (2 + 4 * (DP / 16)) * 64 * sizeof(float);
     const size_t lds = ring > merge ? ring : merge;
+    if (lds > 160 * 1024) return hipErrorNotSupported;
     if (lds > 48 * 1024) {
-        if (const hipError_t e = ensure_lds_limit<&attention_kernel<DP, MASK, DC, NKQ>>(); e != hipSuccess) return e;
+        if (const hipError_t e = ensure_lds_limit<&attention_kernel<DP, MK, DC, NKQ>>(); e != hipSuccess) return e;
     }
     const unsigned qb = (unsigned)((g.q_len + AT_BQ - 1) / AT_BQ);
-    hipLaunchKernelGGL((attention_kernel<DP, MASK, DC, NKQ>), dim3(qb, (unsigned)stacks, (unsigned)g.splits), dim3(256 * NKQ), lds, st, g);
+    hipLaunchKernelGGL((attention_kernel<DP, MK, DC, NKQ>), dim3(qb, (unsigned)stacks, (unsigned)g.splits), dim3(256 * NKQ), lds, st, g);
     if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (g.splits > 1) {
         hipLaunchKernelGGL((attention_merge_kernel<DP>), dim3(qb, (unsigned)stacks), dim3(256), 0, st, g);
@@ -709,18 +768,26 @@ template <int DP, bool MASK, int DC, int NKQ> static hipError_t launch_attention
 // head_dim 80, eight / sixteen wavefronts: 512 keys 10.0 / 10.7 us, 1024: 15.1 / 15.1, 1536: 21.3 / 20.1, 4096: 43.6 / 41.6;
 // 6 heads x 1500 x 1500 x 64 (Whisper): 17.8 / 15.8; 32 x 2048 x 2048 x 96 causal: 78.3 / 71.8
 RT_TUNABLE(g_attention_wide_from, 1280);
+RT_TUNABLE(g_attention_mask_direct, 0); // non-zero: a mask tensor is always read from memory where it is used (for comparisons)
 
-template <int DP, bool MASK, int DC> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
-    if constexpr (DP <= 96) {
-        if (g.splits == 1 && g.kv_len >= g_attention_wide_from) return launch_attention_k<DP, MASK, DC, 4>(g, stacks, st);
+template <int DP, int MK, int DC> static hipError_t launch_attention_dm(const AttnArgs &g, int stacks, hipStream_t st) {
+    if constexpr (DP <= 96 && MK != 2) {
+        if (g.splits == 1 && g.kv_len >= g_attention_wide_from) return launch_attention_k<DP, MK, DC, 4>(g, stacks, st);
     }
-    return launch_attention_k<DP, MASK, DC, 2>(g, stacks, st);
+    return launch_attention_k<DP, MK, DC, 2>(g, stacks, st);
 }
 
 // the kernel built for this head_dim (Whisper 64, Phi-2 80, Phi-3 96, Llama-class 128), else the one that takes it as an argument
 template <int DP, int DC> static hipError_t launch_attention_dp(const AttnArgs &g, int stacks, hipStream_t st) {
-    if (g.D == DC) return g.mask ? launch_attention_dm<DP, true, DC>(g, stacks, st) : launch_attention_dm<DP, false, DC>(g, stacks, st);
-    return g.mask ? launch_attention_dm<DP, true, 0>(g, stacks, st) : launch_attention_dm<DP, false, 0>(g, stacks, st);
+    // a mask tensor whose rows are whole 16-byte vectors travels through the ring; any other is read where it is used
+    const int64_t mrb = g.mask_rs * (g.mask_f32 ? 4 : 2);
+    const int mk = !g.mask ? 0 : ((((uintptr_t)g.mask & 15u) == 0 && mrb % 16 == 0 && mrb >= 16 && mrb < (int64_t(1) << 31) && !g_attention_mask_direct) ? 2 : 1);
+    if (g.D == DC) {
+        if (mk == 2) return launch_attention_dm<DP, 2, DC>(g, stacks, st);
+        return mk ? launch_attention_dm<DP, 1, DC>(g, stacks, st) : launch_attention_dm<DP, 0, DC>(g, stacks, st);
+    }
+    if (mk == 2) return launch_attention_dm<DP, 2, 0>(g, stacks, st);
+    return mk ? launch_attention_dm<DP, 1, 0>(g, stacks, st) : launch_attention_dm<DP, 0, 0>(g, stacks, st);
 }
 
 static int attention_dp(int head_dim) { return head_dim <= 64 ? 64 : (head_dim <= 96 ? 96 : 128); }
