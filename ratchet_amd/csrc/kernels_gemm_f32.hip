@@ -35,6 +35,7 @@ struct GemmF32Args {
     int64_t b_bs, b_ks, b_js; // one of b_ks, b_js is 1
     int64_t o_bs, o_is, o_js;
     int has_bias, bias_on_rows, act;
+    int nt_out; // row-major output whose rows are whole 128-byte lines: written with non-temporal stores
 };
 
 constexpr int F32_BK = 32;
@@ -193,8 +194,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
     float *out = g.out + s * g.o_bs;
     const int64_t iw = i0 + wi * WM, jw = j0 + wj * WN; // this wavefront's corner
     if constexpr (OJ) {
-        // acc[a][b][r] is C[iw + 16 a + fr][jw + 16 b + 4 fq + r]: 16 bytes per lane along a row (non-temporal:
-        // the output is written once), 64 contiguous bytes per row and instruction
+        // acc[a][b][r] is C[iw + 16 a + fr][jw + 16 b + 4 fq + r]: 16 bytes per lane along a row, 64 contiguous bytes per row
+        // and instruction.  Non-temporal (the output is written once) where those 64 bytes are half of a line the next
+        // instruction completes; with rows that do not start on a line (Whisper's scores, 1500 columns: 6000 bytes) the
+        // pieces straddle lines and streaming them costs more than caching them (48 against 31 us at 6 x [1500 x 64] . [64 x 1500])
         rt_with_act(g.act, [&](auto has_act) {
 #pragma unroll
             for (int a = 0; a < TM; a++) {
@@ -215,7 +218,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args g) {
                     }
 #pragma unroll
                     for (int r = 0; r < 4; r++) v[r] = rt_act_k<decltype(has_act)::value>(v[r]);
-                    __builtin_nontemporal_store(v, (float4_t *)(out + i * g.o_is + j));
+                    if (g.nt_out) __builtin_nontemporal_store(v, (float4_t *)(out + i * g.o_is + j));
+                    else *(float4_t *)(out + i * g.o_is + j) = v;
                 }
             }
         });
@@ -295,6 +299,7 @@ hipError_t launch_gemm_f32(const Problem &p, const void *A, const void *B, const
     g.b_bs = p.b_bs, g.b_ks = p.b_ks, g.b_js = p.b_js;
     g.o_bs = p.o_bs, g.o_is = p.o_is, g.o_js = p.o_js;
     g.has_bias = p.has_bias, g.bias_on_rows = p.bias_on_rows, g.act = p.act;
+    g.nt_out = p.o_js == 1 && (p.o_is * 4) % 128 == 0 && (p.o_bs * 4) % 128 == 0 && ((uintptr_t)out & 127u) == 0;
     // 32-row tiles put about three workgroups on a compute unit, whose prologues and epilogues then
     // overlap with each other's MFMAs: better while the fixed costs weigh (26.3 against 28.2 us at
     // K = 384); 96-row tiles read less LDS per MFMA and win from K of about 1000 on (78 against 81 us at 1536).
@@ -307,6 +312,8 @@ hipError_t launch_gemm_f32(const Problem &p, const void *A, const void *B, const
     if (p.K <= 128 && tiles128 >= 2 * (int64_t)dev.num_cus) bm = 128;
     if (g_gemm_f32_bm == 32 || g_gemm_f32_bm == 96 || g_gemm_f32_bm == 128) bm = g_gemm_f32_bm;
     if (bm == 128) return b_kcont ? launch_f32<128, 128, true>(g, p.stacks, stream) : launch_f32<128, 128, false>(g, p.stacks, stream);
+    // up to 64 columns (P . V over a head dimension of 64): 64-column tiles, not two thirds of 96
+    if (bm == 32 && p.N <= 64) return b_kcont ? launch_f32<32, 64, true>(g, p.stacks, stream) : launch_f32<32, 64, false>(g, p.stacks, stream);
     if (bm == 32) return b_kcont ? launch_f32<32, 96, true>(g, p.stacks, stream) : launch_f32<32, 96, false>(g, p.stacks, stream);
     return b_kcont ? launch_f32<96, 96, true>(g, p.stacks, stream) : launch_f32<96, 96, false>(g, p.stacks, stream);
 }

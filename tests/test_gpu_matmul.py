@@ -999,7 +999,10 @@ def test_f32_contiguous_operands(device, oracle):
               (3, 200, 96, 800), (1, 96, 4000, 32),
               # K that is not a whole number of 32-wide tiles (any multiple of 4): the head dimension of 80 of the
               # phi2 / whisper score product q.matmul(k.permute([0, 1, 3, 2]), false, false), shorter than a tile, ragged
-              (32, 512, 512, 80), (2, 100, 64, 4), (1, 60, 120, 20), (2, 129, 200, 100), (1, 96, 96, 36), (1, 300, 52, 1000)]
+              (32, 512, 512, 80), (2, 100, 64, 4), (1, 60, 120, 20), (2, 129, 200, 100), (1, 96, 96, 36), (1, 300, 52, 1000),
+              # Whisper's two attention products (whisper/mha.rs:105-124) at a third of its 1500 positions: output rows that do
+              # not start on a cache line, and 64 output columns
+              (2, 500, 500, 64), (2, 500, 64, 500)]
     for i, (S, M, N, K) in enumerate(shapes):
         rng = np.random.default_rng(1000 + i)
         a = (rng.standard_normal((S, M, K)) * 0.1).astype(np.float32)
